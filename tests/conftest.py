@@ -1,0 +1,22 @@
+"""pytest configuration: registers the ``gpu`` marker and puts the repository
+root on ``sys.path`` so ``come_amd`` and ``oracle`` import from the tree."""
+
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(autouse=True)
+def _seed():
+    import torch
+
+    torch.manual_seed(42)
