@@ -1,0 +1,26 @@
+// Library-wide pieces of the C ABI: version and the per-thread error message.
+#include "come_common.h"
+
+#include <string>
+
+namespace come {
+namespace {
+thread_local std::string g_last_error;
+}
+
+void set_error(const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+}
+
+void clear_error() { g_last_error.clear(); }
+
+}  // namespace come
+
+extern "C" int come_version(void) { return 100; }
+
+extern "C" const char *come_last_error(void) { return come::g_last_error.c_str(); }

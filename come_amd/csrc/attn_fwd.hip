@@ -1,0 +1,371 @@
+// Forward attention over packed variable-length sequences with an additive per-key
+// bias, head_dim 64, for gfx950 (wave64, v_mfma_f32_32x32x16 bf16/f16).
+//
+// Work decomposition
+//   One workgroup (4 wavefronts) owns kBlockM = 128 * QT consecutive queries of one
+//   (segment, head); every wavefront owns QT tiles of 32 queries and walks all keys of
+//   the segment in tiles of 64.  K and V tiles are staged once per workgroup in LDS
+//   (double buffered, one barrier per tile); Q stays in registers.
+//
+// Orientation
+//   Scores are produced transposed, S^T = K' Q'^T, so that in the MFMA accumulator
+//   layout a lane holds ONE query (lane % 32) and 16 keys per 32x32 tile: the row max
+//   and row sum of the online softmax are in-lane reductions plus one exchange between
+//   lane l and lane l ^ 32.  The same registers, rounded to 16 bit, are the B operand
+//   of O^T += V^T P^T without any data movement; V^T fragments come out of the
+//   row-major V tile with the transposing LDS read ds_read_b64_tr_b16.
+//
+// Bias and tail masking without vector ALU work
+//   K' = [K | t_hi t_mid t_lo 0...] (80 columns) and Q' = [Q | 1 1 1 0...] where
+//   t = float(bias) / softmax_scale split exactly into three 16-bit terms, so the
+//   fifth k-step of the score MFMA adds bias / scale to every score (the reference
+//   adds the same quantity, flash_fwd_kernel.h:30-55).  Keys beyond the end of the
+//   segment get t_hi = -inf, which makes their scores -inf and their probabilities 0.
+#include "come_common.h"
+
+namespace come {
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kHeadDim = 64;
+constexpr int kBlockN = 64;          // keys per tile
+constexpr int kKPitch = 88;          // elements per K' row in LDS (64 + 16 bias/zero + 8 pad): 176 B, odd multiple of 16 B
+constexpr int kVPitch = 96;          // elements per V row in LDS: 192 B = 48 banks, 4 rows tile the 64 banks
+constexpr int kThreads = 256;
+
+struct AttnArgs {
+    const uint16_t *q, *k, *v;
+    const uint16_t *bias;            // may be null
+    uint16_t *out;
+    float *lse;                      // may be null
+    const int32_t *cu;
+    int64_t q_rs, q_hs, k_rs, k_hs, v_rs, v_hs, o_rs, o_hs;
+    int64_t total;
+    int n_heads, n_mblocks;
+    float scale, scale_log2, inv_scale;
+};
+
+template <int DT> struct Elem;
+template <> struct Elem<COME_BF16> {
+    static constexpr uint32_t kOne = 0x3F80u, kNegInf = 0xFF80u;
+    __device__ static inline float to_f32(uint16_t x) { return __uint_as_float(static_cast<uint32_t>(x) << 16); }
+    __device__ static inline uint16_t from_f32(float x) { return static_cast<uint16_t>(pack2_bf16(x, 0.f) & 0xffffu); }
+    __device__ static inline uint32_t pack2(float lo, float hi) { return pack2_bf16(lo, hi); }
+    __device__ static inline f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+template <> struct Elem<COME_F16> {
+    static constexpr uint32_t kOne = 0x3C00u, kNegInf = 0xFC00u;
+    __device__ static inline float to_f32(uint16_t x) { return __half2float(__builtin_bit_cast(__half, x)); }
+    __device__ static inline uint16_t from_f32(float x) { return __builtin_bit_cast(uint16_t, __float2half_rn(x)); }
+    __device__ static inline uint32_t pack2(float lo, float hi) { return pack2_f16(lo, hi); }
+    __device__ static inline f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+
+__device__ inline u32x4 zero4() { return u32x4{0u, 0u, 0u, 0u}; }
+
+// exchange between lane l and lane l ^ 32: returns {value of the lower half lane, value of the upper half lane}
+__device__ inline float max_across_halves(float x) {
+    const uint32_t u = __float_as_uint(x);
+    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ inline float sum_across_halves(float x) {
+    const uint32_t u = __float_as_uint(x);
+    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+__device__ inline s16x4 lds_read_tr(const uint16_t *p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(p));
+}
+
+template <int DT, int QT>
+__global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnArgs a) {
+    using E = Elem<DT>;
+    constexpr int kBlockM = 128 * QT;
+    __shared__ __attribute__((aligned(16))) uint16_t lds_k[2][kBlockN * kKPitch];
+    __shared__ __attribute__((aligned(16))) uint16_t lds_v[2][kBlockN * kVPitch];
+
+    // ---- which (segment, head, query block): consecutive blocks of one (segment, head)
+    //      run on the same XCD (workgroup i is dispatched to XCD i % 8) and share K/V in its L2
+    const int n_wg = gridDim.x;
+    int wid = blockIdx.x;
+    const int per_xcd = n_wg >> 3;
+    if (wid < (per_xcd << 3)) wid = (wid & 7) * per_xcd + (wid >> 3);
+    const int mblk = wid % a.n_mblocks;
+    const int rest = wid / a.n_mblocks;
+    const int head = rest % a.n_heads;
+    const int seq = rest / a.n_heads;
+    const int seq_start = a.cu[seq];
+    const int L = a.cu[seq + 1] - seq_start;
+    const int q0 = mblk * kBlockM;
+    if (q0 >= L) return;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int h = lane >> 5;          // which half of the wavefront
+    const int r = lane & 31;          // query column / key row inside a 32x32 tile
+
+    // ---- Q fragments (B operand: n = query r, k = head-dim 16 * ks + 8 * h .. + 7)
+    u32x4 qf[QT][4];
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const int row = q0 + (wave * QT + qt) * 32 + r;
+        const uint16_t *qp = a.q + static_cast<int64_t>(seq_start + min(row, L - 1)) * a.q_rs + head * a.q_hs + 8 * h;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) qf[qt][ks] = *reinterpret_cast<const u32x4 *>(qp + 16 * ks);
+    }
+    // fifth k-step of Q': ones against the three bias terms (lower half), zeros elsewhere
+    const u32x4 q_ext = h == 0 ? u32x4{E::kOne | (E::kOne << 16), E::kOne, 0u, 0u} : zero4();
+
+    // ---- staging of one K'/V tile: thread -> (row sr and sr + 32, 16-byte chunk sc)
+    const int sc = tid & 7;
+    const int sr = tid >> 3;
+    const uint16_t *k_base = a.k + static_cast<int64_t>(seq_start) * a.k_rs + head * a.k_hs + sc * 8;
+    const uint16_t *v_base = a.v + static_cast<int64_t>(seq_start) * a.v_rs + head * a.v_hs + sc * 8;
+    const uint16_t *b_base = a.bias ? a.bias + seq_start : nullptr;
+
+    u32x4 k_stage[2], v_stage[2], b_stage;
+    auto fetch = [&](int n0) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int key = n0 + sr + 32 * i;
+            const bool ok = key < L;
+            k_stage[i] = ok ? *reinterpret_cast<const u32x4 *>(k_base + static_cast<int64_t>(key) * a.k_rs) : zero4();
+            v_stage[i] = ok ? *reinterpret_cast<const u32x4 *>(v_base + static_cast<int64_t>(key) * a.v_rs) : zero4();
+        }
+        if (tid < kBlockN) {
+            const int key = n0 + tid;
+            uint32_t t_hi = E::kNegInf, t_mid = 0, t_lo = 0;
+            if (key < L) {
+                const float t = b_base ? E::to_f32(b_base[key]) * a.inv_scale : 0.f;
+                t_hi = E::from_f32(t);
+                const float hi_f = E::to_f32(static_cast<uint16_t>(t_hi));
+                if (fabsf(hi_f) != INFINITY) {                               // an infinite bias stays a single term
+                    const float r1 = t - hi_f;
+                    t_mid = E::from_f32(r1);
+                    t_lo = E::from_f32(r1 - E::to_f32(static_cast<uint16_t>(t_mid)));
+                }
+            }
+            b_stage = u32x4{t_hi | (t_mid << 16), t_lo, 0u, 0u};
+        }
+    };
+    auto commit = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            *reinterpret_cast<u32x4 *>(&lds_k[buf][(sr + 32 * i) * kKPitch + sc * 8]) = k_stage[i];
+            *reinterpret_cast<u32x4 *>(&lds_v[buf][(sr + 32 * i) * kVPitch + sc * 8]) = v_stage[i];
+        }
+        if (tid < kBlockN) {
+            *reinterpret_cast<u32x4 *>(&lds_k[buf][tid * kKPitch + 64]) = b_stage;
+            *reinterpret_cast<u32x4 *>(&lds_k[buf][tid * kKPitch + 72]) = zero4();
+        }
+    };
+
+    // ---- running state per query tile
+    f32x16 o_acc[QT][2];
+    float m_run[QT], l_run[QT];
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o_acc[qt][dt][i] = 0.f;
+        m_run[qt] = -INFINITY;
+        l_run[qt] = 0.f;
+    }
+
+    const int n_tiles = (L + kBlockN - 1) / kBlockN;
+    fetch(0);
+    commit(0);
+    __syncthreads();
+
+    // LDS read offsets of this lane
+    const int k_off = r * kKPitch + 8 * h;                                   // + 32*mt*pitch + 16*ks
+    const int v_off = (4 * h + ((lane & 15) >> 2)) * kVPitch + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+    for (int j = 0; j < n_tiles; ++j) {
+        const int buf = j & 1;
+        const bool more = j + 1 < n_tiles;
+        if (more) fetch((j + 1) * kBlockN);
+
+        // ---- S^T = K' Q'^T : [64 keys] x [32 * QT queries]
+        f32x16 s_acc[QT][2];
+        const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < 5; ++ks) {
+            const u32x4 kf0 = *reinterpret_cast<const u32x4 *>(&lds_k[buf][k_off + 16 * ks]);
+            const u32x4 kf1 = *reinterpret_cast<const u32x4 *>(&lds_k[buf][k_off + 32 * kKPitch + 16 * ks]);
+#pragma unroll
+            for (int qt = 0; qt < QT; ++qt) {
+                const u32x4 qb = ks < 4 ? qf[qt][ks < 4 ? ks : 0] : q_ext;
+                s_acc[qt][0] = E::mfma(kf0, qb, ks == 0 ? zero16 : s_acc[qt][0]);
+                s_acc[qt][1] = E::mfma(kf1, qb, ks == 0 ? zero16 : s_acc[qt][1]);
+            }
+        }
+
+        // ---- online softmax, in the exp2 domain
+        u32x4 p_frag[QT][4];                                                  // P^T as B operand, one per 16-key step
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+            float mx = s_acc[qt][0][0];
+#pragma unroll
+            for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s_acc[qt][0][i]);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[qt][1][i]);
+            mx = max_across_halves(mx);
+            const float m_new = fmaxf(m_run[qt], mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;            // row fully masked so far
+            const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_use) * a.scale_log2);
+            const float mc = m_use * a.scale_log2;
+            float sum = 0.f;
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[qt][mt][i], a.scale_log2, -mc));
+                    s_acc[qt][mt][i] = p;
+                    sum += p;
+                }
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    u32x4 f;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) f[w] = E::pack2(s_acc[qt][mt][8 * t + 2 * w], s_acc[qt][mt][8 * t + 2 * w + 1]);
+                    p_frag[qt][2 * mt + t] = f;
+                }
+            }
+            l_run[qt] = l_run[qt] * alpha + sum;
+            if (__any(m_new != m_run[qt])) {                                  // rescale O only when some row max moved
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) o_acc[qt][dt][i] *= alpha;
+            }
+            m_run[qt] = m_new;
+        }
+
+        // ---- O^T += V^T P^T
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt) {
+                const uint16_t *vp = &lds_v[buf][v_off + (16 * u) * kVPitch + 32 * dt];
+                const s16x4 lo = lds_read_tr(vp);
+                const s16x4 hi = lds_read_tr(vp + 8 * kVPitch);
+                const u32x2 lo2 = __builtin_bit_cast(u32x2, lo);
+                const u32x2 hi2 = __builtin_bit_cast(u32x2, hi);
+                const u32x4 vf = u32x4{lo2[0], lo2[1], hi2[0], hi2[1]};
+#pragma unroll
+                for (int qt = 0; qt < QT; ++qt) o_acc[qt][dt] = E::mfma(vf, p_frag[qt][u], o_acc[qt][dt]);
+            }
+        }
+
+        if (more) commit(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: normalise, write O (and LSE)
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const float l_tot = sum_across_halves(l_run[qt]);
+        const float inv = 1.0f / l_tot;
+        const int row = q0 + (wave * QT + qt) * 32 + r;
+        if (row < L) {
+            uint16_t *op = a.out + static_cast<int64_t>(seq_start + row) * a.o_rs + head * a.o_hs + 4 * h;
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    u32x2 w;
+                    w[0] = E::pack2(o_acc[qt][dt][4 * g] * inv, o_acc[qt][dt][4 * g + 1] * inv);
+                    w[1] = E::pack2(o_acc[qt][dt][4 * g + 2] * inv, o_acc[qt][dt][4 * g + 3] * inv);
+                    *reinterpret_cast<u32x2 *>(op + 32 * dt + 8 * g) = w;
+                }
+            if (h == 0 && a.lse)
+                a.lse[static_cast<int64_t>(head) * a.total + seq_start + row] = m_run[qt] * a.scale + __logf(l_tot);
+        }
+    }
+}
+
+}  // namespace
+}  // namespace come
+
+using namespace come;
+
+extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v, int dtype, int64_t q_row_stride,
+                                    int64_t q_head_stride, int64_t k_row_stride, int64_t k_head_stride,
+                                    int64_t v_row_stride, int64_t v_head_stride, const int32_t *cu_seqlens,
+                                    int64_t n_seq, int64_t total, int64_t n_heads, int64_t head_dim,
+                                    const void *perkey_bias, int64_t max_seqlen, float softmax_scale, void *out,
+                                    int64_t o_row_stride, int64_t o_head_stride, float *lse, void *stream) {
+    clear_error();
+    COME_REQUIRE(dtype == COME_BF16 || dtype == COME_F16, COME_ERR_UNSUPPORTED,
+                 "come_attn_varlen_fwd: only fp16 and bf16 are supported");
+    COME_REQUIRE(head_dim == kHeadDim, COME_ERR_UNSUPPORTED,
+                 "come_attn_varlen_fwd: only head_dim == 64 is implemented (got %lld)", (long long)head_dim);
+    COME_REQUIRE(n_seq > 0, COME_ERR_INVALID, "come_attn_varlen_fwd: batch size must be positive");
+    COME_REQUIRE(total >= 0 && n_heads > 0 && max_seqlen >= 0, COME_ERR_INVALID,
+                 "come_attn_varlen_fwd: negative size");
+    COME_REQUIRE(total < (1ll << 31) && n_heads < 65536 && n_seq < (1ll << 24), COME_ERR_UNSUPPORTED,
+                 "come_attn_varlen_fwd: problem too large");
+    COME_REQUIRE(softmax_scale > 0.f && softmax_scale < INFINITY, COME_ERR_INVALID,
+                 "come_attn_varlen_fwd: softmax_scale must be positive and finite");
+    if (total == 0 || max_seqlen == 0) return COME_OK;
+    COME_REQUIRE(q && k && v && out && cu_seqlens, COME_ERR_INVALID, "come_attn_varlen_fwd: NULL tensor");
+    const int64_t strides[8] = {q_row_stride, q_head_stride, k_row_stride, k_head_stride,
+                                v_row_stride, v_head_stride, o_row_stride, o_head_stride};
+    for (int i = 0; i < 8; ++i)
+        COME_REQUIRE(strides[i] >= kHeadDim || (i % 2 == 1 && n_heads == 1), COME_ERR_INVALID,
+                     "come_attn_varlen_fwd: stride %d is smaller than head_dim", i);
+    for (int i = 0; i < 6; ++i)
+        COME_REQUIRE(strides[i] % 8 == 0, COME_ERR_UNSUPPORTED,
+                     "come_attn_varlen_fwd: q/k/v strides must be multiples of 8 elements (16-byte loads)");
+    COME_REQUIRE(o_row_stride % 4 == 0 && o_head_stride % 4 == 0, COME_ERR_UNSUPPORTED,
+                 "come_attn_varlen_fwd: out strides must be multiples of 4 elements");
+    COME_REQUIRE((reinterpret_cast<uintptr_t>(q) & 15) == 0 && (reinterpret_cast<uintptr_t>(k) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(v) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0,
+                 COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: q/k/v must be 16-byte aligned, out 8-byte aligned");
+
+    constexpr int QT = 2;
+    constexpr int kBlockM = 128 * QT;
+    AttnArgs a{};
+    a.q = static_cast<const uint16_t *>(q);
+    a.k = static_cast<const uint16_t *>(k);
+    a.v = static_cast<const uint16_t *>(v);
+    a.bias = static_cast<const uint16_t *>(perkey_bias);
+    a.out = static_cast<uint16_t *>(out);
+    a.lse = lse;
+    a.cu = cu_seqlens;
+    a.q_rs = q_row_stride; a.q_hs = q_head_stride;
+    a.k_rs = k_row_stride; a.k_hs = k_head_stride;
+    a.v_rs = v_row_stride; a.v_hs = v_head_stride;
+    a.o_rs = o_row_stride; a.o_hs = o_head_stride;
+    a.total = total;
+    a.n_heads = static_cast<int>(n_heads);
+    a.n_mblocks = static_cast<int>(ceil_div(max_seqlen, kBlockM));
+    a.scale = softmax_scale;
+    a.scale_log2 = softmax_scale * 1.4426950408889634f;
+    a.inv_scale = 1.0f / softmax_scale;
+    const int64_t n_wg = n_seq * n_heads * a.n_mblocks;
+    COME_REQUIRE(n_wg < (1ll << 31), COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: grid too large");
+    const dim3 grid(static_cast<unsigned>(n_wg)), block(kThreads);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == COME_BF16)
+        hipLaunchKernelGGL((attn_fwd_kernel<COME_BF16, QT>), grid, block, 0, s, a);
+    else
+        hipLaunchKernelGGL((attn_fwd_kernel<COME_F16, QT>), grid, block, 0, s, a);
+    COME_CHECK_LAUNCH("come_attn_varlen_fwd");
+    return COME_OK;
+}

@@ -1,0 +1,512 @@
+// Token merge / unmerge for gfx950: HBM-bound gather-mean and gather kernels.
+//
+// Data movement is organised in 16-byte chunks: one thread owns one chunk column of
+// one window (or of one copied token), issues all of the window's loads back to back
+// (nine independent 16-byte loads for a 3x3 window) and writes either their mean
+// (merged) or the rows themselves (kept).  A wavefront therefore reads 1 KiB
+// contiguous per source row and writes 1 KiB contiguous per packed row.
+#include "come_common.h"
+
+namespace come {
+namespace {
+
+constexpr int kThreads = 256;
+
+struct MergeGeom {
+    int rows, n_tok, start, groups;
+    int gh, gw, G;          // window shape, tokens per window
+    int H, W, mw;           // token grid, windows per grid row
+    int cov_h, cov_w;       // part of the grid covered by full windows
+    int tail;               // grid positions outside the full windows
+    int64_t out_rows;
+};
+
+struct MergeArgs {
+    MergeGeom g;
+    const void *tokens;
+    void *out;
+    const uint8_t *mask;
+    const int32_t *offsets;
+    const int32_t *prefix;
+    int64_t *rev64;
+    int32_t *rev32;
+    float *weight;
+    int32_t *count;
+    int64_t group_items;     // rows * groups * chunks (or * chans in the scalar kernel)
+    int64_t group_blocks;    // blocks that own group items
+    int64_t single_items;    // rows * (start + tail) * chunks
+    int chunks;              // 16-byte chunks per token row (vector kernel) / chans (scalar kernel)
+};
+
+__device__ inline void note_row(const MergeArgs &a, int64_t src_flat, int64_t dst) {
+    if (a.rev64) a.rev64[src_flat] = dst;
+    if (a.rev32) a.rev32[src_flat] = static_cast<int32_t>(dst);
+}
+__device__ inline void note_weight(const MergeArgs &a, int64_t dst, int n) {
+    if (dst >= a.g.out_rows) return;
+    if (a.weight) a.weight[dst] = static_cast<float>(n);
+    if (a.count) a.count[dst] = n;
+}
+
+// position `r` (0-based) among the grid positions outside the full windows, image row-major
+__device__ inline int leftover_position(const MergeGeom &g, int r) {
+    const int side = g.W - g.cov_w;                 // leftover columns of a covered grid row
+    const int upper = g.cov_h * side;
+    if (r < upper) {
+        const int y = r / side;
+        return y * g.W + g.cov_w + (r - y * side);
+    }
+    return g.cov_h * g.W + (r - upper);
+}
+
+// ---------------------------------------------------------------------------------
+// bookkeeping: mask -> per-window prefix, per-row length, row offsets   (one workgroup)
+// ---------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void merge_plan_kernel(const uint8_t *__restrict__ mask, int rows, int groups,
+                                                          int start, int G, int tail,
+                                                          int32_t *__restrict__ offsets,
+                                                          int32_t *__restrict__ prefix) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n_waves = blockDim.x >> 6;
+    const uint64_t below = (1ull << lane) - 1ull;
+
+    for (int b = wave; b < rows; b += n_waves) {
+        int running = 0;                                    // wave-uniform
+        for (int m0 = 0; m0 < groups; m0 += 64) {
+            const int m = m0 + lane;
+            const bool valid = m < groups;
+            const bool merged = valid && mask[static_cast<int64_t>(b) * groups + m] != 0;
+            const uint64_t merged_bits = __ballot(merged);
+            const int merged_before = __popcll(merged_bits & below);
+            if (valid) prefix[static_cast<int64_t>(b) * groups + m] = running + merged_before + (lane - merged_before) * G;
+            const int n_valid = min(64, groups - m0);
+            const int n_merged = __popcll(merged_bits);
+            running += n_merged + (n_valid - n_merged) * G;
+        }
+        if (lane == 0) offsets[b + 1] = start + tail + running;
+    }
+    if (threadIdx.x == 0) offsets[0] = 0;
+    __syncthreads();
+
+    if (wave == 0) {                                        // in-place inclusive scan of the row lengths
+        int carry = 0;
+        for (int r0 = 0; r0 < rows; r0 += 64) {
+            const int r = r0 + lane;
+            int v = r < rows ? offsets[r + 1] : 0;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int t = __shfl_up(v, d);
+                if (lane >= d) v += t;
+            }
+            if (r < rows) offsets[r + 1] = v + carry;
+            carry += __shfl(v, 63);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// merge, 16-byte path.  GH x GW fixed at compile time (0 x 0 = run-time window shape).
+// ---------------------------------------------------------------------------------
+template <int DT, int GH, int GW>
+__global__ __launch_bounds__(kThreads) void merge_vec_kernel(const MergeArgs a) {
+    using V = Vec16<DT>;
+    const MergeGeom &g = a.g;
+    const uint4 *__restrict__ src = static_cast<const uint4 *>(a.tokens);
+    uint4 *__restrict__ dst = static_cast<uint4 *>(a.out);
+    const int chunks = a.chunks;
+
+    if (static_cast<int64_t>(blockIdx.x) < a.group_blocks) {
+        const int64_t id = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+        if (id >= a.group_items) return;
+        const int64_t gm = id / chunks;                     // flat (row, window)
+        const int chunk = static_cast<int>(id - gm * chunks);
+        const int b = static_cast<int>(gm / g.groups);
+        const int m = static_cast<int>(gm - static_cast<int64_t>(b) * g.groups);
+        const int wy = m / g.mw;
+        const int wx = m - wy * g.mw;
+        const bool merged = a.mask[gm] != 0;
+        const int64_t row0 = static_cast<int64_t>(a.offsets[b]) + g.start + a.prefix[gm];
+        const int64_t tok0 = static_cast<int64_t>(b) * g.n_tok + g.start + (wy * g.gh) * g.W + wx * g.gw;
+        const uint4 *p = src + tok0 * chunks + chunk;
+
+        if constexpr (GH > 0) {
+            uint4 v[GH * GW];
+#pragma unroll
+            for (int dy = 0; dy < GH; ++dy)
+#pragma unroll
+                for (int dx = 0; dx < GW; ++dx)
+                    v[dy * GW + dx] = p[(static_cast<int64_t>(dy) * g.W + dx) * chunks];
+            if (merged) {
+                float acc[V::N];
+#pragma unroll
+                for (int e = 0; e < V::N; ++e) acc[e] = 0.f;
+#pragma unroll
+                for (int t = 0; t < GH * GW; ++t) {
+                    float f[V::N];
+                    V::unpack(v[t], f);
+#pragma unroll
+                    for (int e = 0; e < V::N; ++e) acc[e] += f[e];
+                }
+#pragma unroll
+                for (int e = 0; e < V::N; ++e) acc[e] = acc[e] / static_cast<float>(GH * GW);
+                if (row0 < g.out_rows) dst[row0 * chunks + chunk] = V::pack(acc);
+            } else {
+#pragma unroll
+                for (int t = 0; t < GH * GW; ++t)
+                    if (row0 + t < g.out_rows) dst[(row0 + t) * chunks + chunk] = v[t];
+            }
+        } else {
+            if (merged) {
+                float acc[V::N];
+#pragma unroll
+                for (int e = 0; e < V::N; ++e) acc[e] = 0.f;
+                for (int dy = 0; dy < g.gh; ++dy) {
+#pragma unroll 4
+                    for (int dx = 0; dx < g.gw; ++dx) {
+                        float f[V::N];
+                        V::unpack(p[(static_cast<int64_t>(dy) * g.W + dx) * chunks], f);
+#pragma unroll
+                        for (int e = 0; e < V::N; ++e) acc[e] += f[e];
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < V::N; ++e) acc[e] = acc[e] / static_cast<float>(g.G);
+                if (row0 < g.out_rows) dst[row0 * chunks + chunk] = V::pack(acc);
+            } else {
+                int64_t r = row0;
+                for (int dy = 0; dy < g.gh; ++dy) {
+#pragma unroll 4
+                    for (int dx = 0; dx < g.gw; ++dx, ++r)
+                        if (r < g.out_rows) dst[r * chunks + chunk] = p[(static_cast<int64_t>(dy) * g.W + dx) * chunks];
+                }
+            }
+        }
+
+        if (chunk == 0) {                                   // index map and counts of this window
+            int t = 0;
+            for (int dy = 0; dy < g.gh; ++dy)
+                for (int dx = 0; dx < g.gw; ++dx, ++t)
+                    note_row(a, tok0 + static_cast<int64_t>(dy) * g.W + dx, merged ? row0 : row0 + t);
+            if (merged) {
+                note_weight(a, row0, g.G);
+            } else {
+                for (int t2 = 0; t2 < g.G; ++t2) note_weight(a, row0 + t2, 1);
+            }
+        }
+        return;
+    }
+
+    // copied tokens: specials in front, leftover grid positions behind the windows
+    const int64_t id = (static_cast<int64_t>(blockIdx.x) - a.group_blocks) * kThreads + threadIdx.x;
+    if (id >= a.single_items) return;
+    const int per_row = g.start + g.tail;
+    const int64_t t = id / chunks;
+    const int chunk = static_cast<int>(id - t * chunks);
+    const int b = static_cast<int>(t / per_row);
+    const int j = static_cast<int>(t - static_cast<int64_t>(b) * per_row);
+    int tok;
+    int64_t row;
+    if (j < g.start) {
+        tok = j;
+        row = static_cast<int64_t>(a.offsets[b]) + j;
+    } else {
+        const int r = j - g.start;
+        tok = g.start + leftover_position(g, r);
+        row = static_cast<int64_t>(a.offsets[b + 1]) - g.tail + r;
+    }
+    const int64_t flat = static_cast<int64_t>(b) * g.n_tok + tok;
+    if (row < g.out_rows) dst[row * chunks + chunk] = src[flat * chunks + chunk];
+    if (chunk == 0) {
+        note_row(a, flat, row);
+        note_weight(a, row, 1);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// merge, element path: any channel count / alignment (e.g. the 2-channel position
+// tensor).  One thread per (window, channel) or (copied token, channel).
+// ---------------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(kThreads) void merge_elem_kernel(const MergeArgs a) {
+    using V = Vec16<DT>;
+    const MergeGeom &g = a.g;
+    const int chans = a.chunks;
+
+    if (static_cast<int64_t>(blockIdx.x) < a.group_blocks) {
+        const int64_t id = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+        if (id >= a.group_items) return;
+        const int64_t gm = id / chans;
+        const int c = static_cast<int>(id - gm * chans);
+        const int b = static_cast<int>(gm / g.groups);
+        const int m = static_cast<int>(gm - static_cast<int64_t>(b) * g.groups);
+        const int wy = m / g.mw;
+        const int wx = m - wy * g.mw;
+        const bool merged = a.mask[gm] != 0;
+        const int64_t row0 = static_cast<int64_t>(a.offsets[b]) + g.start + a.prefix[gm];
+        const int64_t tok0 = static_cast<int64_t>(b) * g.n_tok + g.start + (wy * g.gh) * g.W + wx * g.gw;
+        float acc = 0.f;
+        int t = 0;
+        for (int dy = 0; dy < g.gh; ++dy) {
+            for (int dx = 0; dx < g.gw; ++dx, ++t) {
+                const int64_t tok = tok0 + static_cast<int64_t>(dy) * g.W + dx;
+                const float x = V::load1(a.tokens, tok * chans + c);
+                if (merged) {
+                    acc += x;
+                } else if (row0 + t < g.out_rows) {
+                    V::store1(a.out, (row0 + t) * chans + c, x);
+                }
+                if (c == 0) {
+                    note_row(a, tok, merged ? row0 : row0 + t);
+                    if (!merged) note_weight(a, row0 + t, 1);
+                }
+            }
+        }
+        if (merged) {
+            if (row0 < g.out_rows) V::store1(a.out, row0 * chans + c, acc / static_cast<float>(g.G));
+            if (c == 0) note_weight(a, row0, g.G);
+        }
+        return;
+    }
+
+    const int64_t id = (static_cast<int64_t>(blockIdx.x) - a.group_blocks) * kThreads + threadIdx.x;
+    if (id >= a.single_items) return;
+    const int per_row = g.start + g.tail;
+    const int64_t t = id / chans;
+    const int c = static_cast<int>(id - t * chans);
+    const int b = static_cast<int>(t / per_row);
+    const int j = static_cast<int>(t - static_cast<int64_t>(b) * per_row);
+    int tok;
+    int64_t row;
+    if (j < g.start) {
+        tok = j;
+        row = static_cast<int64_t>(a.offsets[b]) + j;
+    } else {
+        const int r = j - g.start;
+        tok = g.start + leftover_position(g, r);
+        row = static_cast<int64_t>(a.offsets[b + 1]) - g.tail + r;
+    }
+    const int64_t flat = static_cast<int64_t>(b) * g.n_tok + tok;
+    if (row < g.out_rows) V::store1(a.out, row * chans + c, V::load1(a.tokens, flat * chans + c));
+    if (c == 0) {
+        note_row(a, flat, row);
+        note_weight(a, row, 1);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// unmerge: out[i, :] = merged[rev[i], :]
+// ---------------------------------------------------------------------------------
+constexpr int kSplitRows = 4;      // output rows per thread (independent loads in flight)
+
+template <typename IndexT>
+__global__ __launch_bounds__(kThreads) void split_vec_kernel(const uint4 *__restrict__ merged, int64_t merged_rows,
+                                                             const IndexT *__restrict__ rev, int64_t total,
+                                                             int chunks, uint4 *__restrict__ out, int64_t items) {
+    const int64_t id = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (id >= items) return;
+    const int64_t quad = id / chunks;
+    const int chunk = static_cast<int>(id - quad * chunks);
+    const int64_t i0 = quad * kSplitRows;
+    uint4 v[kSplitRows];
+#pragma unroll
+    for (int r = 0; r < kSplitRows; ++r) {
+        v[r] = make_uint4(0, 0, 0, 0);
+        if (i0 + r < total) {
+            const int64_t s = static_cast<int64_t>(rev[i0 + r]);
+            if (s >= 0 && s < merged_rows) v[r] = merged[s * chunks + chunk];
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < kSplitRows; ++r)
+        if (i0 + r < total) out[(i0 + r) * chunks + chunk] = v[r];
+}
+
+template <typename IndexT>
+__global__ __launch_bounds__(kThreads) void split_elem_kernel(const uint8_t *__restrict__ merged, int64_t merged_rows,
+                                                              const IndexT *__restrict__ rev, int64_t total,
+                                                              int64_t row_bytes, int elem_bytes,
+                                                              uint8_t *__restrict__ out) {
+    const int64_t id = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const int64_t per_row = row_bytes / elem_bytes;
+    if (id >= total * per_row) return;
+    const int64_t i = id / per_row;
+    const int64_t c = id - i * per_row;
+    const int64_t s = static_cast<int64_t>(rev[i]);
+    const bool ok = s >= 0 && s < merged_rows;
+    if (elem_bytes == 4) {
+        reinterpret_cast<uint32_t *>(out)[i * per_row + c] =
+            ok ? reinterpret_cast<const uint32_t *>(merged)[s * per_row + c] : 0u;
+    } else {
+        reinterpret_cast<uint16_t *>(out)[i * per_row + c] =
+            ok ? reinterpret_cast<const uint16_t *>(merged)[s * per_row + c] : uint16_t(0);
+    }
+}
+
+template <int DT>
+void launch_merge_vec(const MergeArgs &a, int64_t blocks, hipStream_t stream) {
+    const MergeGeom &g = a.g;
+    const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+#define COME_MERGE_CASE(GH_, GW_)                                                              \
+    if (g.gh == GH_ && g.gw == GW_) {                                                          \
+        hipLaunchKernelGGL((merge_vec_kernel<DT, GH_, GW_>), grid, block, 0, stream, a);       \
+        return;                                                                                \
+    }
+    COME_MERGE_CASE(3, 3)
+    COME_MERGE_CASE(2, 2)
+    COME_MERGE_CASE(1, 2)
+    COME_MERGE_CASE(1, 4)
+    COME_MERGE_CASE(1, 8)
+    COME_MERGE_CASE(1, 9)
+#undef COME_MERGE_CASE
+    hipLaunchKernelGGL((merge_vec_kernel<DT, 0, 0>), grid, block, 0, stream, a);
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+}  // namespace come
+
+using namespace come;
+
+extern "C" int come_merge_plan(const uint8_t *merge_mask, int64_t rows, int64_t groups, int64_t start_index,
+                               int64_t group_size, int64_t tail, int32_t *offsets, int32_t *group_prefix,
+                               void *stream) {
+    clear_error();
+    COME_REQUIRE(rows >= 0 && groups >= 0, COME_ERR_INVALID, "come_merge_plan: rows/groups must be >= 0");
+    COME_REQUIRE(start_index >= 0, COME_ERR_INVALID, "come_merge_plan: start_index must be >= 0");
+    COME_REQUIRE(group_size > 0, COME_ERR_INVALID, "come_merge_plan: group_size must be > 0");
+    COME_REQUIRE(tail >= 0, COME_ERR_INVALID, "come_merge_plan: tail must be >= 0");
+    COME_REQUIRE(offsets != nullptr, COME_ERR_INVALID, "come_merge_plan: offsets is NULL");
+    COME_REQUIRE(rows * groups == 0 || (merge_mask && group_prefix), COME_ERR_INVALID,
+                 "come_merge_plan: merge_mask / group_prefix is NULL");
+    const int64_t n_tok = start_index + groups * group_size + tail;
+    COME_REQUIRE(rows < (1ll << 31) && groups < (1ll << 31) && rows * n_tok < (1ll << 31), COME_ERR_UNSUPPORTED,
+                 "come_merge_plan: rows * tokens per row must stay below 2^31");
+    hipLaunchKernelGGL(merge_plan_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream), merge_mask,
+                       static_cast<int>(rows), static_cast<int>(groups), static_cast<int>(start_index),
+                       static_cast<int>(group_size), static_cast<int>(tail), offsets, group_prefix);
+    COME_CHECK_LAUNCH("come_merge_plan");
+    return COME_OK;
+}
+
+extern "C" int come_token_merge(const void *tokens, int dtype, int64_t rows, int64_t n_tok, int64_t chans,
+                                int64_t start_index, int64_t group_h, int64_t group_w, int64_t grid_h,
+                                int64_t grid_w, const uint8_t *merge_mask, const int32_t *offsets,
+                                const int32_t *group_prefix, void *out, int64_t out_rows, int64_t *rev_i64,
+                                int32_t *rev_i32, float *weight_f32, int32_t *count_i32, void *stream) {
+    clear_error();
+    COME_REQUIRE(dtype_ok(dtype), COME_ERR_UNSUPPORTED, "come_token_merge: unsupported dtype %d", dtype);
+    COME_REQUIRE(rows >= 0 && n_tok >= 0 && chans >= 1 && out_rows >= 0, COME_ERR_INVALID,
+                 "come_token_merge: negative size or chans < 1");
+    COME_REQUIRE(start_index >= 0, COME_ERR_INVALID, "come_token_merge: start_index must be >= 0");
+    COME_REQUIRE(group_h > 0 && group_w > 0, COME_ERR_INVALID, "come_token_merge: group_h and group_w must be > 0");
+    COME_REQUIRE(grid_h >= 0 && grid_w >= 0, COME_ERR_INVALID, "come_token_merge: grid_h / grid_w must be >= 0");
+    COME_REQUIRE(n_tok == start_index + grid_h * grid_w, COME_ERR_INVALID,
+                 "come_token_merge: N != start_index + grid_h * grid_w (%lld != %lld + %lld * %lld)",
+                 (long long)n_tok, (long long)start_index, (long long)grid_h, (long long)grid_w);
+    COME_REQUIRE(rows * n_tok < (1ll << 31) && chans < (1ll << 24), COME_ERR_UNSUPPORTED,
+                 "come_token_merge: rows * tokens per row must stay below 2^31");
+    if (rows == 0 || n_tok == 0) return COME_OK;
+    COME_REQUIRE(tokens && out && offsets, COME_ERR_INVALID, "come_token_merge: tokens / out / offsets is NULL");
+
+    MergeArgs a{};
+    MergeGeom &g = a.g;
+    g.rows = static_cast<int>(rows);
+    g.n_tok = static_cast<int>(n_tok);
+    g.start = static_cast<int>(start_index);
+    g.gh = static_cast<int>(group_h);
+    g.gw = static_cast<int>(group_w);
+    g.G = g.gh * g.gw;
+    g.H = static_cast<int>(grid_h);
+    g.W = static_cast<int>(grid_w);
+    g.mw = g.W / g.gw;
+    const int mh = g.H / g.gh;
+    g.groups = mh * g.mw;
+    g.cov_h = mh * g.gh;
+    g.cov_w = g.mw * g.gw;
+    g.tail = g.H * g.W - g.cov_h * g.cov_w;
+    if (g.groups == 0) {            // no full window: every grid position is a leftover, row-major
+        g.cov_h = 0;
+        g.cov_w = 0;
+        g.mw = 1;
+    }
+    g.out_rows = out_rows;
+    COME_REQUIRE(g.groups == 0 || (merge_mask && group_prefix), COME_ERR_INVALID,
+                 "come_token_merge: merge_mask / group_prefix is NULL");
+    a.tokens = tokens;
+    a.out = out;
+    a.mask = merge_mask;
+    a.offsets = offsets;
+    a.prefix = group_prefix;
+    a.rev64 = rev_i64;
+    a.rev32 = rev_i32;
+    a.weight = weight_f32;
+    a.count = count_i32;
+
+    const int64_t row_bytes = chans * dtype_bytes(dtype);
+    const bool vec = (row_bytes % 16 == 0) && aligned16(tokens) && aligned16(out);
+    a.chunks = static_cast<int>(vec ? row_bytes / 16 : chans);
+    a.group_items = rows * g.groups * a.chunks;
+    a.group_blocks = ceil_div(a.group_items, kThreads);
+    a.single_items = rows * (g.start + g.tail) * a.chunks;
+    const int64_t blocks = a.group_blocks + ceil_div(a.single_items, kThreads);
+    COME_REQUIRE(blocks < (1ll << 31), COME_ERR_UNSUPPORTED, "come_token_merge: problem too large for one launch");
+    if (blocks == 0) return COME_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (vec) {
+        if (dtype == COME_BF16) launch_merge_vec<COME_BF16>(a, blocks, s);
+        else if (dtype == COME_F16) launch_merge_vec<COME_F16>(a, blocks, s);
+        else launch_merge_vec<COME_F32>(a, blocks, s);
+    } else {
+        const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+        if (dtype == COME_BF16) hipLaunchKernelGGL(merge_elem_kernel<COME_BF16>, grid, block, 0, s, a);
+        else if (dtype == COME_F16) hipLaunchKernelGGL(merge_elem_kernel<COME_F16>, grid, block, 0, s, a);
+        else hipLaunchKernelGGL(merge_elem_kernel<COME_F32>, grid, block, 0, s, a);
+    }
+    COME_CHECK_LAUNCH("come_token_merge");
+    return COME_OK;
+}
+
+extern "C" int come_token_split(const void *merged, int dtype, int64_t merged_rows, int64_t chans,
+                                const int64_t *rev_i64, const int32_t *rev_i32, int64_t total, void *out,
+                                void *stream) {
+    clear_error();
+    COME_REQUIRE(dtype_ok(dtype), COME_ERR_UNSUPPORTED, "come_token_split: unsupported dtype %d", dtype);
+    COME_REQUIRE(merged_rows >= 0 && chans >= 1 && total >= 0, COME_ERR_INVALID,
+                 "come_token_split: negative size or chans < 1");
+    COME_REQUIRE((rev_i64 != nullptr) != (rev_i32 != nullptr) || total == 0, COME_ERR_INVALID,
+                 "come_token_split: exactly one of rev_i64 / rev_i32 must be given");
+    if (total == 0) return COME_OK;
+    COME_REQUIRE(out != nullptr && (merged != nullptr || merged_rows == 0), COME_ERR_INVALID,
+                 "come_token_split: merged / out is NULL");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t row_bytes = chans * dtype_bytes(dtype);
+    const bool vec = (row_bytes % 16 == 0) && aligned16(merged) && aligned16(out);
+    if (vec) {
+        const int chunks = static_cast<int>(row_bytes / 16);
+        const int64_t items = ceil_div(total, kSplitRows) * chunks;
+        const int64_t blocks = ceil_div(items, kThreads);
+        COME_REQUIRE(blocks < (1ll << 31), COME_ERR_UNSUPPORTED, "come_token_split: problem too large for one launch");
+        const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+        if (rev_i64)
+            hipLaunchKernelGGL(split_vec_kernel<int64_t>, grid, block, 0, s, static_cast<const uint4 *>(merged),
+                               merged_rows, rev_i64, total, chunks, static_cast<uint4 *>(out), items);
+        else
+            hipLaunchKernelGGL(split_vec_kernel<int32_t>, grid, block, 0, s, static_cast<const uint4 *>(merged),
+                               merged_rows, rev_i32, total, chunks, static_cast<uint4 *>(out), items);
+    } else {
+        const int eb = dtype_bytes(dtype);
+        const int64_t blocks = ceil_div(total * chans, kThreads);
+        COME_REQUIRE(blocks < (1ll << 31), COME_ERR_UNSUPPORTED, "come_token_split: problem too large for one launch");
+        const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+        if (rev_i64)
+            hipLaunchKernelGGL(split_elem_kernel<int64_t>, grid, block, 0, s, static_cast<const uint8_t *>(merged),
+                               merged_rows, rev_i64, total, row_bytes, eb, static_cast<uint8_t *>(out));
+        else
+            hipLaunchKernelGGL(split_elem_kernel<int32_t>, grid, block, 0, s, static_cast<const uint8_t *>(merged),
+                               merged_rows, rev_i32, total, row_bytes, eb, static_cast<uint8_t *>(out));
+    }
+    COME_CHECK_LAUNCH("come_token_split");
+    return COME_OK;
+}

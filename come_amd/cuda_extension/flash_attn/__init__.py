@@ -1,0 +1,82 @@
+"""Python surface of the forward-only varlen attention, mirroring
+``src/cuda_extension/flash_attn/__init__.py:21-33, 235-295, 439-477`` of the reference:
+``flash_attn_varlen_qkvpacked_func``, ``flash_attn_varlen_qkvpacked_func_w_perkey_bias`` and
+``infer_flash_attn_varlen_max_seqlen`` with the same arguments, defaults and return values.
+Calling backward raises ``RuntimeError`` (forward-only build, as in the reference).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import flash_attn_fwd_cuda as _C
+
+__all__ = [
+    "flash_attn_varlen_qkvpacked_func",
+    "flash_attn_varlen_qkvpacked_func_w_perkey_bias",
+    "infer_flash_attn_varlen_max_seqlen",
+]
+
+
+def infer_flash_attn_varlen_max_seqlen(cu_seqlens: torch.Tensor) -> int:
+    """Longest segment of ``cu_seqlens`` as a Python int (one host sync); 0 during ONNX export."""
+    if torch.onnx.is_in_onnx_export():
+        return 0
+    return int((cu_seqlens[1:] - cu_seqlens[:-1]).max().item())
+
+
+def _pad_head(t: torch.Tensor, head_size: int) -> torch.Tensor:
+    if head_size % 8 != 0:
+        return torch.nn.functional.pad(t, [0, 8 - head_size % 8])
+    return t
+
+
+class _VarlenQKVPacked(torch.autograd.Function):
+    """Shared forward of the plain and the biased operator (``perkey_bias`` may be None)."""
+
+    @staticmethod
+    def forward(ctx, qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale, causal, window_size,
+                softcap, alibi_slopes, deterministic, return_softmax, is_grad_enabled, op_name):
+        ctx.op_name = op_name
+        if softmax_scale is None:
+            softmax_scale = qkv.shape[-1] ** (-0.5)
+        if len(window_size) != 2:
+            raise ValueError(f"window_size must contain 2 values, got {window_size}")
+        q, k, v = qkv[:, 0].detach(), qkv[:, 1].detach(), qkv[:, 2].detach()
+        head_size_og = q.size(2)
+        q, k, v = (_pad_head(t, head_size_og) for t in (q, k, v))
+        args = (q, k, v, None, cu_seqlens, cu_seqlens, None, None, None, alibi_slopes)
+        tail = (max_seqlen, max_seqlen, dropout_p, softmax_scale, False, causal, int(window_size[0]),
+                int(window_size[1]), softcap, return_softmax and dropout_p > 0, None)
+        if perkey_bias is None:
+            out_padded, softmax_lse, s_dmask, rng_state = _C.varlen_fwd(*args, *tail)
+        else:
+            out_padded, softmax_lse, s_dmask, rng_state = _C.varlen_fwd_w_perkey_bias(*args, perkey_bias, *tail)
+        ctx.mark_non_differentiable(softmax_lse, s_dmask, rng_state)
+        out = out_padded[..., :head_size_og]
+        return out if not return_softmax else (out, softmax_lse, s_dmask)
+
+    @staticmethod
+    def backward(ctx, *args):
+        raise RuntimeError(f"{ctx.op_name} backward is not supported in this forward-only build.")
+
+
+def flash_attn_varlen_qkvpacked_func(qkv, cu_seqlens, max_seqlen, dropout_p=0.0, softmax_scale=None, causal=False,
+                                     window_size=(-1, -1), softcap=0.0, alibi_slopes=None, deterministic=False,
+                                     return_attn_probs=False):
+    """``qkv [total, 3, nheads, headdim]``, ``cu_seqlens [batch + 1] int32`` -> ``out [total, nheads, headdim]``
+    (plus ``softmax_lse [nheads, total]`` and an empty tensor when ``return_attn_probs``)."""
+    return _VarlenQKVPacked.apply(qkv, cu_seqlens, max_seqlen, None, dropout_p, softmax_scale, causal, window_size,
+                                  softcap, alibi_slopes, deterministic, return_attn_probs, torch.is_grad_enabled(),
+                                  "flash_attn_varlen_qkvpacked_func")
+
+
+def flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p=0.0,
+                                                   softmax_scale=None, causal=False, window_size=(-1, -1),
+                                                   softcap=0.0, alibi_slopes=None, deterministic=False,
+                                                   return_attn_probs=False):
+    """Same as :func:`flash_attn_varlen_qkvpacked_func` with ``softmax(Q K^T * scale + perkey_bias[key]) V``;
+    ``perkey_bias [total]`` has the dtype of ``qkv`` and is indexed like the packed keys."""
+    return _VarlenQKVPacked.apply(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale, causal,
+                                  window_size, softcap, alibi_slopes, deterministic, return_attn_probs,
+                                  torch.is_grad_enabled(), "flash_attn_varlen_qkvpacked_func_w_perkey_bias")

@@ -1,0 +1,139 @@
+"""``varlen_fwd`` / ``varlen_fwd_w_perkey_bias`` on the HIP attention kernel.
+
+Positional signatures and return lists follow the reference's pybind module
+``flash_attn_fwd_cuda`` (``src/cuda_extension/flash_attn/flash_api.cpp:538-607``,
+checks ``:291-408``, bias checks ``:274-288``).  Only what the Co-Me call sites
+reach is implemented: fp16 / bf16, head_dim 64, self-attention over one set of
+``cu_seqlens``, no causal mask, no dropout, no alibi / softcap / sliding window /
+paged KV / left padding.  Anything else raises ``RuntimeError`` instead of
+computing something different.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ... import _lib
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _unsupported(cond: bool, what: str) -> None:
+    if cond:
+        raise RuntimeError(f"come_amd flash-attention: {what} is not supported by this forward-only HIP build")
+
+
+def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
+                     perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal,
+                     window_size_left, window_size_right, softcap, return_softmax, gen):
+    _check(q.dtype in (torch.float16, torch.bfloat16), "FlashAttention only support fp16 and bf16 data type")
+    _check(k.dtype == q.dtype, "query and key must have the same dtype")
+    _check(v.dtype == q.dtype, "query and value must have the same dtype")
+    _check(cu_seqlens_q.dtype == torch.int32, "cu_seqlens_q must have dtype int32")
+    _check(cu_seqlens_k.dtype == torch.int32, "cu_seqlens_k must have dtype int32")
+    for name, t in (("q", q), ("k", k), ("v", v), ("cu_seqlens_q", cu_seqlens_q), ("cu_seqlens_k", cu_seqlens_k)):
+        _check(t.is_cuda, f"{name} must be on CUDA")
+    _check(q.stride(-1) == 1 and k.stride(-1) == 1 and v.stride(-1) == 1,
+           "Input tensor must have contiguous last dimension")
+    _check(cu_seqlens_q.is_contiguous() and cu_seqlens_k.is_contiguous(), "cu_seqlens must be contiguous")
+    _check(q.dim() == 3 and k.dim() == 3 and v.dim() == 3, "q, k, v must be [total, nheads, headdim]")
+
+    _unsupported(block_table is not None, "paged KV (block_table)")
+    _unsupported(seqused_k is not None, "seqused_k")
+    _unsupported(leftpad_k is not None, "leftpad_k")
+    _unsupported(alibi_slopes is not None, "alibi_slopes")
+    _unsupported(p_dropout != 0.0, "dropout")
+    _unsupported(softcap != 0.0, "softcap")
+    _unsupported(return_softmax, "return_softmax")
+    max_seqlen_q, max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
+    if max_seqlen_q == 1:
+        is_causal = False
+    _unsupported(bool(is_causal), "causal masking")
+    if window_size_left >= max_seqlen_k:
+        window_size_left = -1
+    if window_size_right >= max_seqlen_k:
+        window_size_right = -1
+    _unsupported(window_size_left >= 0 or window_size_right >= 0, "sliding-window attention")
+
+    batch_size = cu_seqlens_q.numel() - 1
+    total_q, num_heads, head_size = q.shape
+    total_k, num_heads_k, _ = k.shape
+    _check(batch_size > 0, "batch size must be positive")
+    _check(head_size <= 256, "FlashAttention forward only supports head dimension at most 256")
+    _check(head_size % 8 == 0, "query, key, value, and out_ must have a head_size that is a multiple of 8")
+    _check(num_heads % num_heads_k == 0, "Number of heads in key/value must divide number of heads in query")
+    _check(tuple(k.shape) == (total_k, num_heads_k, head_size), "k must have shape (total_k, num_heads_k, head_size)")
+    _check(tuple(v.shape) == (total_k, num_heads_k, head_size), "v must have shape (total_k, num_heads_k, head_size)")
+    _check(tuple(cu_seqlens_k.shape) == (batch_size + 1,), "cu_seqlens_k must have shape (batch_size + 1)")
+    _unsupported(num_heads != num_heads_k, "grouped-query attention (num_heads != num_heads_k)")
+    _unsupported(head_size != 64, f"head_dim {head_size} (only 64 is implemented)")
+    _unsupported(total_q != total_k or max_seqlen_q != max_seqlen_k
+                 or (cu_seqlens_q.data_ptr() != cu_seqlens_k.data_ptr() and not torch.equal(cu_seqlens_q, cu_seqlens_k)),
+                 "cross attention (different query and key packing)")
+
+    dev = q.device
+    if perkey_bias is not None:
+        _check(perkey_bias.dtype == q.dtype,
+               f"perkey_bias dtype must match QKV dtype ({q.dtype}), got {perkey_bias.dtype}")
+        _check(perkey_bias.is_cuda, "perkey_bias must be on CUDA")
+        _check(perkey_bias.is_contiguous(), "perkey_bias must be contiguous")
+        _check(tuple(perkey_bias.shape) == (total_k,),
+               f"perkey_bias must have shape (total_k,), got {tuple(perkey_bias.shape)}")
+
+    def _aligned(t):          # the kernel issues 16-byte loads
+        return t.data_ptr() % 16 == 0 and t.stride(0) % 8 == 0 and t.stride(1) % 8 == 0
+    q, k, v = (t if _aligned(t) else t.contiguous() for t in (q, k, v))
+
+    with torch.cuda.device(dev):
+        if out_ is not None:
+            out = out_
+            _check(out.dtype == q.dtype, "Output must have the same dtype as inputs")
+            _check(out.is_cuda, "out must be on CUDA")
+            _check(out.stride(-1) == 1, "Output tensor must have contiguous last dimension")
+            _check(tuple(out.shape) == (total_q, num_heads, head_size), "out has the wrong shape")
+        else:
+            out = torch.empty((total_q, num_heads, head_size), dtype=q.dtype, device=dev)
+        softmax_lse = torch.empty((num_heads, total_q), dtype=torch.float32, device=dev)
+        p = torch.empty((0,), dtype=q.dtype, device=dev)
+        rng_state = torch.empty((2,), dtype=torch.int64, device=dev)
+        if zero_tensors:
+            out.zero_()
+            softmax_lse.fill_(-math.inf)
+        if max_seqlen_k > 0:
+            lib = _lib.load()
+            _lib.check(lib.come_attn_varlen_fwd(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.dtype_code(q.dtype),
+                q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
+                cu_seqlens_q.data_ptr(), batch_size, total_q, num_heads, head_size,
+                _lib.ptr(perkey_bias), max_seqlen_k, float(softmax_scale),
+                out.data_ptr(), out.stride(0), out.stride(1), softmax_lse.data_ptr(), _lib.current_stream(dev)))
+        else:
+            out.zero_()
+            softmax_lse.fill_(math.inf)
+    return [out, softmax_lse, p, rng_state]
+
+
+def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
+               max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal,
+               window_size_left, window_size_right, softcap, return_softmax, gen=None):
+    """Forward pass (variable length).  Returns ``[out, softmax_lse, p, rng_state]``."""
+    return _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table,
+                            alibi_slopes, None, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
+                            zero_tensors, is_causal, window_size_left, window_size_right, softcap,
+                            return_softmax, gen)
+
+
+def varlen_fwd_w_perkey_bias(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table,
+                             alibi_slopes, perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
+                             zero_tensors, is_causal, window_size_left, window_size_right, softcap,
+                             return_softmax, gen=None):
+    """Forward pass (variable length) with a per-key additive bias."""
+    return _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table,
+                            alibi_slopes, perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
+                            zero_tensors, is_causal, window_size_left, window_size_right, softcap,
+                            return_softmax, gen)

@@ -1,0 +1,173 @@
+/*
+ * come_hip.h — C ABI of libcome_hip.so, the MI355X (gfx950) implementation of the
+ * Co-Me accelerated-inference hot path: confidence-guided token merge, unmerge and
+ * the forward varlen attention with an additive per-key bias.
+ *
+ * Every entry point takes plain device pointers and sizes, enqueues its kernels on
+ * the HIP stream passed in `stream` (a hipStream_t; NULL = the null stream) and
+ * returns without synchronising.  Nothing here allocates device memory: outputs and
+ * small work buffers are supplied by the caller.  The device that owns the pointers
+ * must be the current HIP device of the calling thread.
+ *
+ * Return value: COME_OK (0) or a come_status error code; come_last_error() then
+ * holds a message for the calling thread.
+ *
+ * Each declaration cites the interface of the reference (co-me-tokens/CoMe, paths
+ * relative to its root) that the entry point stands in for.
+ */
+#ifndef COME_HIP_H
+#define COME_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum come_status {
+    COME_OK = 0,
+    COME_ERR_INVALID = 1,     /* bad argument (null pointer, negative size, inconsistent shape) */
+    COME_ERR_UNSUPPORTED = 2, /* a combination this library does not implement                 */
+    COME_ERR_HIP = 3          /* a HIP runtime call or kernel launch failed                    */
+} come_status;
+
+typedef enum come_dtype {
+    COME_F32 = 0,
+    COME_F16 = 1,
+    COME_BF16 = 2
+} come_dtype;
+
+/* Library version (major * 10000 + minor * 100 + patch). */
+int come_version(void);
+
+/* Message of the last failing call made by this thread ("" if none). */
+const char *come_last_error(void);
+
+/*
+ * come_merge_plan — from the merge mask to packed-row bookkeeping.
+ *
+ *   merge_mask   [rows, groups] bytes, non-zero = merge that group into one row
+ *   offsets      [rows + 1] int32 out: offsets[0] = 0,
+ *                offsets[b+1] - offsets[b] = start_index + tail + sum_m (mask ? 1 : group_size)
+ *   group_prefix [rows, groups] int32 out: exclusive prefix of (mask ? 1 : group_size)
+ *                inside the row
+ *
+ * Stands in for block_prefix_scan_kernel + the cumsum glue of the reference
+ * (src/cuda_extension/co_me/src/kernel_token_merge.cu:12-46, 271-286) and for
+ * `offsets` of func_token_merge (src/accelerate/token_merger/co_me.py:177-182).
+ * `tail` (tokens behind the groups that are always copied) is 0 in the reference.
+ */
+int come_merge_plan(const uint8_t *merge_mask, int64_t rows, int64_t groups,
+                    int64_t start_index, int64_t group_size, int64_t tail,
+                    int32_t *offsets, int32_t *group_prefix, void *stream);
+
+/*
+ * come_token_merge — gather-mean of the selected windows into packed rows.
+ *
+ *   tokens   [rows, n_tok, chans] of `dtype`, contiguous;
+ *            n_tok = start_index + grid_h * grid_w
+ *   windows  group_h x group_w over the grid_h x grid_w token grid, block-row-major,
+ *            row-major inside a window; a 1-D merge of `M` groups of `G` tokens is
+ *            grid_h = 1, grid_w = M * G, group_h = 1, group_w = G.
+ *            Grid positions outside the (grid_h / group_h) x (grid_w / group_w) full
+ *            windows are copied behind the windows in image row-major order.
+ *   merge_mask, offsets, group_prefix   as produced by / passed to come_merge_plan
+ *            (same rows, groups = full windows per row, start_index,
+ *            group_size = group_h * group_w, tail = positions outside full windows)
+ *   out      [out_rows, chans] of `dtype`; rows at or beyond out_rows are not written
+ *   rev_i64 / rev_i32   [rows * n_tok] packed row of every source token, in the
+ *            original (image row-major) token order; either may be NULL
+ *   weight_f32 / count_i32   [out_rows] number of source tokens per packed row;
+ *            either may be NULL
+ *
+ * Packed layout per row block: [specials | window 0 | window 1 | ... | leftover positions];
+ * a merged window is one row = mean of its tokens (fp32 accumulation, one rounding).
+ *
+ * Stands in for co_me_token_merge_cuda (src/cuda_extension/co_me/src/binding.cpp:33-42,
+ * kernel_token_merge.cu:50-191, 239-348), for func_token_merge
+ * (src/accelerate/token_merger/co_me.py:153-222) and, with group_h > 1, for
+ * func_token_merge_2d (src/accelerate/token_merger/co_me_2d.py:174-211) without its
+ * permuted copy of the tokens.
+ */
+int come_token_merge(const void *tokens, int dtype, int64_t rows, int64_t n_tok, int64_t chans,
+                     int64_t start_index, int64_t group_h, int64_t group_w,
+                     int64_t grid_h, int64_t grid_w,
+                     const uint8_t *merge_mask, const int32_t *offsets, const int32_t *group_prefix,
+                     void *out, int64_t out_rows,
+                     int64_t *rev_i64, int32_t *rev_i32, float *weight_f32, int32_t *count_i32,
+                     void *stream);
+
+/*
+ * come_token_split — unmerge: out[i, :] = merged[rev[i], :].
+ *
+ *   merged  [merged_rows, chans] of `dtype`, contiguous
+ *   rev     [total] int64 (rev_i64) or int32 (rev_i32); exactly one is non-NULL
+ *   out     [total, chans] of `dtype`
+ * An index outside [0, merged_rows) yields a row of zeros.
+ *
+ * Stands in for co_me_token_split_cuda (src/cuda_extension/co_me/src/binding.cpp:44-51,
+ * kernel_token_merge.cu:195-233, 354-398) and func_token_split
+ * (src/accelerate/token_merger/co_me.py:241-254).
+ */
+int come_token_split(const void *merged, int dtype, int64_t merged_rows, int64_t chans,
+                     const int64_t *rev_i64, const int32_t *rev_i32, int64_t total,
+                     void *out, void *stream);
+
+/*
+ * come_select_windows — per-window confidence mean and lowest-confidence selection.
+ *
+ *   conf     [batch * frames, grid_h, grid_w] of `dtype` (COME_BF16 or COME_F32), contiguous
+ *   mode     0 = ranking: per batch element, over its frames * windows means jointly,
+ *                mask = mean < quantile(float(mean), threshold) with torch.quantile's
+ *                linear interpolation;
+ *            1 = absolute: mask = mean < threshold
+ *   means_f32 [batch * frames, windows] float out (the means, rounded to `dtype` first);
+ *            may be NULL
+ *   merge_mask [batch * frames, windows] bytes out (1 = merge)
+ *   work     device scratch of at least come_select_work_bytes(...) bytes
+ *
+ * Stands in for the window-mean + torch.quantile + compare sequence of
+ * _CoMe_2D_Base.build_ctx (src/accelerate/token_merger/co_me_2d.py:268-298).
+ */
+int come_select_windows(const void *conf, int dtype, int64_t batch, int64_t frames,
+                        int64_t grid_h, int64_t grid_w, int64_t group_h, int64_t group_w,
+                        int mode, float threshold,
+                        float *means_f32, uint8_t *merge_mask, void *work, int64_t work_bytes,
+                        void *stream);
+int64_t come_select_work_bytes(int64_t batch, int64_t frames, int64_t grid_h, int64_t grid_w,
+                               int64_t group_h, int64_t group_w);
+
+/*
+ * come_attn_varlen_fwd — softmax(Q K^T * softmax_scale + bias[key]) V per packed
+ * segment and head, forward only, no causal mask, no dropout.
+ *
+ *   q, k, v   [total, n_heads, head_dim] views of `dtype` (COME_BF16 or COME_F16) with
+ *             unit stride in the last dimension; *_row_stride / *_head_stride in elements
+ *             (q/k/v are usually slices of one packed [total, 3, n_heads, head_dim] tensor)
+ *   cu_seqlens [n_seq + 1] int32 segment boundaries, cu_seqlens[n_seq] <= total
+ *   perkey_bias [total] of `dtype`, or NULL for plain attention
+ *   max_seqlen  upper bound of the segment lengths (sizes the launch grid)
+ *   out       [total, n_heads, head_dim] of `dtype`, strides in elements
+ *   lse       [n_heads, total] float: logsumexp of the biased, scaled scores; may be NULL
+ * Only head_dim == 64 is implemented.
+ *
+ * Stands in for varlen_fwd / varlen_fwd_w_perkey_bias
+ * (src/cuda_extension/flash_attn/flash_api.cpp:291-607; kernel
+ * src/cuda_extension/flash_attn/src/flash_fwd_kernel.h:30-55, 80-545) as reached from
+ * flash_attn_varlen_qkvpacked_func[_w_perkey_bias]
+ * (src/cuda_extension/flash_attn/__init__.py:235-295, 439-477).
+ */
+int come_attn_varlen_fwd(const void *q, const void *k, const void *v, int dtype,
+                         int64_t q_row_stride, int64_t q_head_stride,
+                         int64_t k_row_stride, int64_t k_head_stride,
+                         int64_t v_row_stride, int64_t v_head_stride,
+                         const int32_t *cu_seqlens, int64_t n_seq, int64_t total,
+                         int64_t n_heads, int64_t head_dim,
+                         const void *perkey_bias, int64_t max_seqlen, float softmax_scale,
+                         void *out, int64_t o_row_stride, int64_t o_head_stride,
+                         float *lse, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COME_HIP_H */

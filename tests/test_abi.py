@@ -1,0 +1,55 @@
+"""CPU-only checks of the C-ABI library: it loads, exports every function the header
+declares, and its argument checks answer without touching a GPU."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from come_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "come_hip.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(come_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_is_built():
+    assert os.path.exists(_lib.LIB_PATH), "run `python -m come_amd.build`"
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    lib = _lib.load()
+    names = _declared_functions()
+    assert len(names) >= 8
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in come_hip.h but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature"
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_version_and_error_string():
+    lib = _lib.load()
+    assert lib.come_version() >= 100
+    # invalid arguments are rejected on the host, before any HIP call
+    assert lib.come_merge_plan(None, 1, 1, -1, 2, 0, None, None, None) == 1
+    assert b"start_index" in lib.come_last_error()
+    assert lib.come_token_merge(None, 7, 1, 1, 1, 0, 1, 1, 1, 1, None, None, None, None, 0,
+                                None, None, None, None, None) == 2
+    assert b"dtype" in lib.come_last_error()
+    assert lib.come_attn_varlen_fwd(None, None, None, _lib.COME_BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 128,
+                                    None, 10, 0.125, None, 64, 64, None, None) == 2
+    assert b"head_dim" in lib.come_last_error()
+    assert lib.come_select_work_bytes(1, 16, 37, 37, 3, 3) >= 16 * 144 * 4
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libcome_hip.so")
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _lib.load()

@@ -1,0 +1,206 @@
+"""GPU parity: forward varlen attention with a per-key bias through the C-ABI library
+against the fp32 closed-form oracle.
+
+Tolerances: the reference's own test uses atol = rtol = 1e-2 per element
+(test_flex_attention_bias.py:20-21); the build target is max-abs <= 1e-2 and
+mean-abs <= 1e-3 in bf16.  Both are asserted.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from come_amd.cuda_extension import (
+    flash_attn_varlen_qkvpacked_func,
+    flash_attn_varlen_qkvpacked_func_w_perkey_bias,
+    infer_flash_attn_varlen_max_seqlen,
+)
+from come_amd.cuda_extension.flash_attn import flash_attn_fwd_cuda
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+MAX_ABS, MEAN_ABS = 1e-2, 1e-3
+
+SEGMENT_SETS = [[32, 48, 24, 24], [56, 49, 23], [128], [60, 40], [50], [128, 256], [100, 150, 50], [64] * 4,
+                [1], [3, 1, 2], [65], [257, 31], [700, 333, 64], [1000]]
+
+
+def _cu(lens):
+    return torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+
+
+def _compare(out, ref):
+    out = out.float().cpu()
+    diff = (out - ref).abs()
+    assert float(diff.max()) <= MAX_ABS, f"max-abs {float(diff.max())}"
+    assert float(diff.mean()) <= MEAN_ABS, f"mean-abs {float(diff.mean())}"
+    torch.testing.assert_close(out, ref, atol=1e-2, rtol=1e-2)
+
+
+def _run(lens, H, dtype, bias_kind="weights", scale=None, return_lse=False):
+    P, D = sum(lens), 64
+    qkv = torch.randn(P, 3, H, D).to(dtype)
+    if bias_kind == "weights":
+        bias = torch.rand(P).clamp(min=1e-3).log().to(dtype)
+    elif bias_kind == "counts":
+        bias = torch.where(torch.rand(P) < 0.3, math.log(9.0), 0.0).to(dtype)
+    else:
+        bias = None
+    cu = _cu(lens)
+    ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias, softmax_scale=scale)
+    args = (qkv.to(DEV), cu.to(DEV), max(lens))
+    if bias is None:
+        res = flash_attn_varlen_qkvpacked_func(*args, softmax_scale=scale, return_attn_probs=return_lse)
+    else:
+        res = flash_attn_varlen_qkvpacked_func_w_perkey_bias(*args, perkey_bias=bias.to(DEV), softmax_scale=scale,
+                                                             return_attn_probs=return_lse)
+    if return_lse:
+        out, lse, _ = res
+        torch.testing.assert_close(lse.cpu(), ref_lse, atol=2e-3, rtol=1e-3)
+    else:
+        out = res
+    assert out.shape == (P, H, D) and out.dtype == dtype
+    _compare(out, ref)
+
+
+@pytest.mark.parametrize("lens", SEGMENT_SETS, ids=[str(s) for s in SEGMENT_SETS])
+def test_bias_matches_closed_form_bf16(lens):
+    _run(lens, H=4, dtype=torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+def test_dtypes(dtype):
+    _run([64, 64], H=4, dtype=dtype)
+    _run([100, 150, 50], H=2, dtype=dtype, bias_kind="counts")
+
+
+@pytest.mark.parametrize("lens", [[128, 256], [300, 77], [2048, 1111]])
+def test_plain_attention_and_lse(lens):
+    _run(lens, H=2, dtype=torch.bfloat16, bias_kind=None, return_lse=True)
+    _run(lens, H=2, dtype=torch.bfloat16, bias_kind="counts", return_lse=True)
+
+
+def test_sixteen_heads_long_segments_and_other_scale():
+    _run([3000, 1500], H=16, dtype=torch.bfloat16, bias_kind="counts")
+    _run([500, 260], H=3, dtype=torch.bfloat16, scale=0.2)           # scale that is not a power of two
+
+
+def test_zero_bias_equals_plain_operator():
+    lens, H = [64, 64], 4
+    P = sum(lens)
+    qkv = torch.randn(P, 3, H, 64, device=DEV).half()
+    cu = _cu(lens).to(DEV)
+    plain = flash_attn_varlen_qkvpacked_func(qkv, cu, 64, softmax_scale=0.125)
+    biased = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, 64, perkey_bias=torch.zeros(P, device=DEV).half(),
+                                                            softmax_scale=0.125)
+    torch.testing.assert_close(plain, biased, atol=1e-4, rtol=1e-4)     # test_flex_attention_bias.py:279-300
+
+
+def test_bias_has_effect():
+    P, H = 128, 2
+    qkv = torch.randn(P, 3, H, 64, device=DEV).half()
+    cu = torch.tensor([0, 128], device=DEV, dtype=torch.int32)
+    zero = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, 128, perkey_bias=torch.zeros(P, device=DEV).half())
+    some = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, 128, perkey_bias=torch.randn(P, device=DEV).half())
+    assert not torch.allclose(zero, some, atol=1e-4)
+
+
+def test_count_bias_equals_key_duplication():
+    L, H, c = 200, 2, 9
+    qkv = torch.randn(L, 3, H, 64).bfloat16()
+    count = torch.ones(L)
+    count[17], count[150] = c, c
+    a = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), _cu([L]).to(DEV), L,
+                                                       perkey_bias=count.log().bfloat16().to(DEV))
+    dup = torch.cat([qkv, qkv[17:18].repeat(c - 1, 1, 1, 1), qkv[150:151].repeat(c - 1, 1, 1, 1)])
+    b = flash_attn_varlen_qkvpacked_func(dup.to(DEV), _cu([dup.shape[0]]).to(DEV), dup.shape[0])
+    # log(9) rounded to bf16 is 2.203125 (exp -> 9.054): the identity holds to that rounding
+    diff = (a.float() - b[:L].float()).abs()
+    assert float(diff.max()) <= 2e-2 and float(diff.mean()) <= 2e-3
+
+
+def test_strided_views_and_separate_tensors():
+    lens, H = [90, 41], 4
+    P = sum(lens)
+    qkv = torch.randn(P, 3, H, 64).bfloat16()
+    bias = torch.randn(P).bfloat16()
+    cu = _cu(lens)
+    ref, _ = oracle.biased_varlen_attention(qkv, cu, bias)
+    q, k, v = (qkv[:, i].contiguous().to(DEV) for i in range(3))      # contiguous [P, H, D] tensors
+    out = flash_attn_fwd_cuda.varlen_fwd_w_perkey_bias(q, k, v, None, cu.to(DEV), cu.to(DEV), None, None, None, None,
+                                                       bias.to(DEV), 90, 90, 0.0, 0.125, False, False, -1, -1, 0.0,
+                                                       False, None)
+    assert len(out) == 4 and out[1].shape == (H, P) and out[1].dtype == torch.float32
+    _compare(out[0], ref)
+    big = torch.zeros(P, 5, H, 72).bfloat16()                          # odd strides: row 5*H*72, head 72
+    big[:, 1:4, :, :64] = qkv
+    out2 = flash_attn_varlen_qkvpacked_func_w_perkey_bias(big.to(DEV)[:, 1:4, :, :64], cu.to(DEV), 90,
+                                                          perkey_bias=bias.to(DEV))
+    _compare(out2, ref)
+
+
+def test_max_seqlen_helper_and_empty_segment():
+    lens = [40, 0, 90]
+    cu = _cu(lens).to(DEV)
+    assert infer_flash_attn_varlen_max_seqlen(cu) == 90
+    P = sum(lens)
+    qkv = torch.randn(P, 3, 2, 64).bfloat16()
+    bias = torch.randn(P).bfloat16()
+    ref, _ = oracle.biased_varlen_attention(qkv, _cu(lens), bias)
+    out = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu, 90, perkey_bias=bias.to(DEV))
+    _compare(out, ref)
+
+
+def test_unsupported_arguments_raise():
+    P = 64
+    cu = torch.tensor([0, 64], device=DEV, dtype=torch.int32)
+    qkv = torch.randn(P, 3, 2, 64, device=DEV).bfloat16()
+    bias = torch.zeros(P, device=DEV).bfloat16()
+    with pytest.raises(RuntimeError, match="causal"):
+        flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, 64, perkey_bias=bias, causal=True)
+    with pytest.raises(RuntimeError, match="dropout"):
+        flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, 64, perkey_bias=bias, dropout_p=0.1)
+    with pytest.raises(RuntimeError, match="head_dim"):
+        flash_attn_varlen_qkvpacked_func(torch.randn(P, 3, 2, 32, device=DEV).half(), cu, 64)
+    with pytest.raises(RuntimeError, match="dtype"):
+        flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, 64, perkey_bias=bias.half())
+    with pytest.raises(RuntimeError, match="shape"):
+        flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, 64, perkey_bias=bias[:10])
+    with pytest.raises(RuntimeError, match="fp16 and bf16"):
+        flash_attn_varlen_qkvpacked_func(qkv.float(), cu, 64)
+    q = qkv.clone().requires_grad_(True)
+    out = flash_attn_varlen_qkvpacked_func_w_perkey_bias(q, cu, 64, perkey_bias=bias)
+    with pytest.raises(RuntimeError, match="backward is not supported"):
+        out.sum().backward()
+
+
+def test_full_size_c3_rows_against_oracle_rows():
+    """BASELINE attention config: 16 heads x 64, two packed sequences of 25 536 and 21 848 tokens,
+    bias = log(count), count in {1, 9}.  The full fp32 oracle is too slow on a CPU at this size, so a
+    sample of query rows is checked against the closed form, plus the logsumexp identity."""
+    H, D = 16, 64
+    lens = [25536, 21848]
+    P = sum(lens)
+    g = torch.Generator().manual_seed(0)
+    qkv = torch.randn(P, 3, H, D, generator=g).bfloat16()
+    count = torch.ones(P)
+    count[torch.randperm(lens[0], generator=g)[:2304]] = 9.0
+    count[lens[0] + torch.randperm(lens[1], generator=g)[:2765]] = 9.0
+    bias = count.log().bfloat16()
+    cu = _cu(lens)
+    out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), max(lens),
+                                                                 perkey_bias=bias.to(DEV), return_attn_probs=True)
+    out, lse = out.float().cpu(), lse.cpu()
+    assert bool(torch.isfinite(out).all())
+    rows = [0, 1, 31, 32, 255, 256, 12345, 25535, 25536, 25537, 30000, P - 1]
+    q, k, v = qkv.float().unbind(1)
+    for row in rows:
+        s, e = (0, lens[0]) if row < lens[0] else (lens[0], P)
+        scores = torch.einsum("hd,khd->hk", q[row], k[s:e]) * 0.125 + bias.float()[None, s:e]
+        ref = torch.einsum("hk,khd->hd", torch.softmax(scores, -1), v[s:e])
+        diff = (out[row] - ref).abs()
+        assert float(diff.max()) <= MAX_ABS and float(diff.mean()) <= MEAN_ABS
+        torch.testing.assert_close(lse[:, row], torch.logsumexp(scores, -1), atol=2e-3, rtol=1e-3)

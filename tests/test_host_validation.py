@@ -1,0 +1,45 @@
+"""Host-side argument checks of the drop-in Python layer (CPU only): the messages are the ones
+the reference's tests match (test_token_merge_func.py:298-318, test_token_merge_2d.py:288-321)."""
+
+import pytest
+import torch
+
+from come_amd.token_merger import func_token_merge, func_token_merge_2d
+from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
+
+
+@pytest.mark.parametrize("tokens,mask,start,G,msg", [
+    (torch.randn(2, 7, 4), torch.ones(2, 3, dtype=torch.bool), 0, 2, "Expected N = start_index"),
+    (torch.randn(2, 6, 4), torch.ones(3, 3, dtype=torch.bool), 0, 2, "merge_mask batch"),
+    (torch.randn(1, 6, 4), torch.ones(1, 3, dtype=torch.bool), -1, 2, "start_index"),
+    (torch.randn(1, 6, 4), torch.ones(1, 3, dtype=torch.bool), 0, 0, "group_size"),
+    (torch.randn(1, 6, 4), torch.ones(1, 3, dtype=torch.float32), 0, 2, "torch.bool"),
+])
+def test_merge_1d_validation(tokens, mask, start, G, msg):
+    with pytest.raises(ValueError, match=msg):
+        func_token_merge(tokens=tokens, merge_mask=mask, start_index=start, group_size=G)
+
+
+@pytest.mark.parametrize("tokens,mask,start,gh,gw,H,W,msg", [
+    (torch.randn(1, 15, 4), torch.ones(1, 3, dtype=torch.bool), 0, 2, 3, 3, 5, "H.*divisible"),
+    (torch.randn(1, 12, 4), torch.ones(1, 2, dtype=torch.bool), 0, 2, 5, 4, 3, "W.*divisible"),
+    (torch.randn(2, 16, 4), torch.ones(3, 4, dtype=torch.bool), 0, 2, 2, 4, 4, "merge_mask batch"),
+    (torch.randn(1, 10, 4), torch.ones(1, 4, dtype=torch.bool), 0, 2, 2, 4, 4, "Expected N"),
+    (torch.randn(1, 16, 4), torch.ones(1, 2, dtype=torch.bool), 0, 2, 2, 4, 4, "Expected M"),
+    (torch.randn(1, 16, 4), torch.ones(1, 4, dtype=torch.bool), -1, 2, 2, 4, 4, "start_index"),
+    (torch.randn(1, 16, 4), torch.ones(1, 4, dtype=torch.bool), 0, 0, 2, 4, 4, "group_h.*group_w.*> 0"),
+    (torch.randn(1, 16, 4), torch.ones(1, 4, dtype=torch.float32), 0, 2, 2, 4, 4, "torch.bool"),
+])
+def test_merge_2d_validation(tokens, mask, start, gh, gw, H, W, msg):
+    with pytest.raises(ValueError, match=msg):
+        func_token_merge_2d(tokens=tokens, merge_mask=mask, start_index=start, group_h=gh, group_w=gw, H=H, W=W)
+
+
+def test_operators_refuse_cpu_tensors():
+    # valid arguments on the CPU must not silently run somewhere else
+    with pytest.raises(RuntimeError, match="CUDA"):
+        func_token_merge(torch.randn(1, 6, 4), 0, 2, torch.ones(1, 3, dtype=torch.bool))
+    qkv = torch.randn(8, 3, 2, 64).bfloat16()
+    cu = torch.tensor([0, 8], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, 8, perkey_bias=torch.zeros(8).bfloat16())
