@@ -1,0 +1,354 @@
+"""Benchmark of the Co-Me hot path on one MI355X.
+
+``python bench.py --gpus 1 --steps K --warmup W`` prints ONE JSON line.
+
+Headline ("step"): one forward pass of the biased varlen attention over the BASELINE
+attention configuration (16 heads x 64, two packed sequences of 25 536 and 21 848 tokens after a
+50 % / 60 % 3x3 merge of 32 frames of 37x37 patches, bias = log(count), bf16).  Its throughput is
+algorithmic flops (sum over segments of 4 L^2 d H) per second.
+
+The same line carries, under ``other``, the merge / unmerge microbenchmark (16 frames of 37x37,
+C = 1024, bf16, 3x3 windows, ratio 0.5) as GB/s of algorithmic bytes with its own roofline, and
+the select + plan + merge pipeline rate.
+
+``roofline`` times the dominant kernel with HIP events on the launch stream; ``cpu_baseline`` times
+the reference's PyTorch CPU path (SDPA with the bias as attn_mask) on a bounded sample of the same
+workload on the host cores.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0       # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
+    ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge"], default=None,
+                    help="run a single kernel in a loop (for profilers); prints a short JSON line")
+    return ap.parse_args()
+
+
+# ------------------------------------------------------------------------------------------
+# synthetic workloads
+# ------------------------------------------------------------------------------------------
+
+def packed_counts(frames: int, windows: int, specials: int, leftover: int, merged_windows: int, gen):
+    """Counts (1 or 9) of one packed sequence in layout order: per frame
+    [specials | windows (one 9 or nine 1s) | leftover positions]; ``merged_windows`` windows are chosen
+    jointly over all frames."""
+    import torch
+
+    chosen = torch.zeros(frames * windows, dtype=torch.bool)
+    chosen[torch.randperm(frames * windows, generator=gen)[:merged_windows]] = True
+    chosen = chosen.reshape(frames, windows)
+    parts = []
+    for f in range(frames):
+        parts.append(torch.ones(specials))
+        w = torch.where(chosen[f][:, None], torch.tensor([9.0] + [0.0] * 8), torch.ones(9)).reshape(-1)
+        parts.append(w[w > 0])
+        parts.append(torch.ones(leftover))
+    return torch.cat(parts)
+
+
+def make_attention_workload(device):
+    import torch
+
+    gen = torch.Generator().manual_seed(0)
+    H, D = 16, 64
+    counts0 = packed_counts(32, 144, 5, 73, 2304, gen)      # ratio 0.50 -> 25 536 tokens
+    counts1 = packed_counts(32, 144, 5, 73, 2765, gen)      # ratio 0.60 -> 21 848 tokens
+    lens = [counts0.numel(), counts1.numel()]
+    assert lens == [25536, 21848], lens
+    P = sum(lens)
+    torch.manual_seed(0)
+    qkv = torch.randn(P, 3, H, D, device=device, dtype=torch.float32).bfloat16()
+    bias = torch.cat([counts0, counts1]).log().bfloat16().to(device)
+    cu = torch.tensor([0, lens[0], P], dtype=torch.int32, device=device)
+    flops = sum(4.0 * L * L * D * H for L in lens)
+    return dict(qkv=qkv, bias=bias, cu=cu, lens=lens, flops=flops, H=H, D=D)
+
+
+def smooth_confidence(frames, H, W, seed):
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    a = torch._standard_gamma(torch.full((frames, H, W), 2.0), generator=g)
+    b = torch._standard_gamma(torch.full((frames, H, W), 5.0), generator=g)
+    x = a / (a + b)                                            # Beta(2, 5)
+    r = 9
+    ker = torch.exp(-torch.arange(-r, r + 1).float() ** 2 / (2 * 3.0 ** 2))
+    ker = ker / ker.sum()
+    y = torch.nn.functional.pad(x[:, None], (r, r, r, r), mode="reflect")
+    y = torch.nn.functional.conv2d(y, ker.view(1, 1, 1, -1))
+    y = torch.nn.functional.conv2d(y, ker.view(1, 1, -1, 1))[:, 0]
+    return 0.5 * x + 0.5 * y
+
+
+# ------------------------------------------------------------------------------------------
+# timed legs
+# ------------------------------------------------------------------------------------------
+
+def time_loop(fn, steps, warmup):
+    """Returns (wall seconds for `steps` calls, HIP-event milliseconds for the same region)."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, start.elapsed_time(stop)
+
+
+def bench_attention(steps, warmup, device):
+    from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
+
+    w = make_attention_workload(device)
+    max_len = max(w["lens"])
+
+    def step():
+        return flash_attn_varlen_qkvpacked_func_w_perkey_bias(w["qkv"], w["cu"], max_len, perkey_bias=w["bias"],
+                                                              softmax_scale=0.125)
+
+    wall, ev_ms = time_loop(step, steps, warmup)
+    return w, wall, ev_ms
+
+
+def merge_workload(device, ratio=0.5, sets=8):
+    """BASELINE merge microbench: 16 frames, 37x37 patches + 5 specials, C = 1024, bf16.  ``sets`` rotating
+    input / output buffer sets keep the working set (> 500 MB) out of the 256 MB Infinity Cache."""
+    import torch
+    from come_amd import _lib
+
+    frames, H, W, S0, C = 16, 37, 37, 5, 1024
+    N = S0 + H * W
+    lib = _lib.load()
+    conf = smooth_confidence(frames, H, W, seed=0).to(device)
+    torch.manual_seed(0)
+    tokens = [torch.randn(frames, N, C, device=device).bfloat16() for _ in range(sets)]
+    M = (H // 3) * (W // 3)
+    tail = H * W - M * 9
+    mask = torch.empty(frames, M, dtype=torch.uint8, device=device)
+    means = torch.empty(frames, M, dtype=torch.float32, device=device)
+    offsets = torch.empty(frames + 1, dtype=torch.int32, device=device)
+    prefix = torch.empty(frames, M, dtype=torch.int32, device=device)
+    stream = _lib.current_stream(device)
+
+    def select_and_plan():
+        _lib.check(lib.come_select_windows(conf.data_ptr(), _lib.COME_F32, 1, frames, H, W, 3, 3, 0, ratio,
+                                           means.data_ptr(), mask.data_ptr(), None, 0, stream))
+        _lib.check(lib.come_merge_plan(mask.data_ptr(), frames, M, S0, 9, tail, offsets.data_ptr(),
+                                       prefix.data_ptr(), stream))
+
+    select_and_plan()
+    P = int(offsets[-1].item())
+    outs = [torch.empty(P, C, dtype=torch.bfloat16, device=device) for _ in range(sets)]
+    index_map = torch.empty(frames * N, dtype=torch.int32, device=device)
+    counts = torch.empty(P, dtype=torch.int32, device=device)
+    restored = [torch.empty(frames * N, C, dtype=torch.bfloat16, device=device) for _ in range(sets)]
+    state = {"i": 0}
+
+    def merge_only():
+        i = state["i"] = (state["i"] + 1) % sets
+        _lib.check(lib.come_token_merge(tokens[i].data_ptr(), _lib.COME_BF16, frames, N, C, S0, 3, 3, H, W,
+                                        mask.data_ptr(), offsets.data_ptr(), prefix.data_ptr(), outs[i].data_ptr(), P,
+                                        None, index_map.data_ptr(), None, counts.data_ptr(), stream))
+
+    def pipeline():
+        select_and_plan()
+        merge_only()
+
+    def split_only():
+        i = state["i"] = (state["i"] + 1) % sets
+        _lib.check(lib.come_token_split(outs[i].data_ptr(), _lib.COME_BF16, P, C, None, index_map.data_ptr(),
+                                        frames * N, restored[i].data_ptr(), stream))
+
+    merge_bytes = frames * N * C * 2 + P * C * 2 + frames * N * 4 + P * 4 + frames * H * W * 4 + (frames + 1) * 4
+    split_bytes = P * C * 2 + frames * N * 4 + frames * N * C * 2
+    return dict(merge_only=merge_only, pipeline=pipeline, split_only=split_only, P=P, merge_bytes=merge_bytes,
+                split_bytes=split_bytes, frames=frames, N=N, C=C, ratio=ratio, tokens=tokens, conf=conf,
+                keep=(outs, restored, index_map, counts, mask, means, offsets, prefix))
+
+
+def bench_merge_unmerge(device, iters=200, warmup=20):
+    w = merge_workload(device)
+    for _ in range(8):
+        w["merge_only"]()                                       # fill every output set before unmerge reads it
+    _, merge_ms = time_loop(w["merge_only"], iters, warmup)
+    _, pipe_ms = time_loop(w["pipeline"], iters, warmup)
+    _, split_ms = time_loop(w["split_only"], iters, warmup)
+    merge_gbs = w["merge_bytes"] / (merge_ms / iters * 1e-3) / 1e9
+    split_gbs = w["split_bytes"] / (split_ms / iters * 1e-3) / 1e9
+    return w, {
+        "merge": {"workload": "C2 merge: 16 frames 37x37+5, C=1024 bf16, 3x3, ratio 0.5, P=%d" % w["P"],
+                  "value": round(merge_gbs, 1), "unit": "GB/s", "us_per_call": round(merge_ms / iters * 1e3, 2),
+                  "algorithmic_bytes": w["merge_bytes"], "iters": iters, "rotating_buffer_sets": 8,
+                  "roofline": {"bound": "hbm", "achieved": round(merge_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                               "frac": round(merge_gbs / PEAK_HBM_GBS, 4), "traffic": None},
+                  "select_plan_merge_us": round(pipe_ms / iters * 1e3, 2)},
+        "unmerge": {"workload": "C2 unmerge: P=%d -> %d rows, C=1024 bf16" % (w["P"], w["frames"] * w["N"]),
+                    "value": round(split_gbs, 1), "unit": "GB/s", "us_per_call": round(split_ms / iters * 1e3, 2),
+                    "algorithmic_bytes": w["split_bytes"], "iters": iters, "rotating_buffer_sets": 8,
+                    "roofline": {"bound": "hbm", "achieved": round(split_gbs, 1), "peak": PEAK_HBM_GBS,
+                                 "unit": "GB/s", "frac": round(split_gbs / PEAK_HBM_GBS, 4), "traffic": None}},
+    }
+
+
+# ------------------------------------------------------------------------------------------
+# host-CPU baseline (the reference's PyTorch path on the CPU), bounded sample
+# ------------------------------------------------------------------------------------------
+
+def cpu_baseline_attention(w, q_rows=2048):
+    """SDPA in bf16 with the bias as attn_mask, the first ``q_rows`` queries of segment 0 against all of
+    its 25 536 keys, all 16 heads.  Same flop formula as the GPU figure (4 * rows * L * d * H)."""
+    import torch
+    import oracle
+
+    cores = os.cpu_count() or 1
+    threads = min(cores, 16)
+    torch.set_num_threads(threads)
+    L = w["lens"][0]
+    qkv = w["qkv"][:L].cpu()
+    bias = w["bias"][:L].cpu()
+    # the oracle's SDPA leg works on whole segments; restrict the queries by packing a view
+    q, k, v = qkv.unbind(1)
+    mask = bias[None, None, None, :]
+    kh, vh = k.transpose(0, 1).unsqueeze(0), v.transpose(0, 1).unsqueeze(0)
+    qh = q[:q_rows].transpose(0, 1).unsqueeze(0)
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        torch.nn.functional.scaled_dot_product_attention(qh, kh, vh, attn_mask=mask, scale=0.125)
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[1]
+    flops = 4.0 * q_rows * L * w["D"] * w["H"]
+    del oracle
+    return {"value": round(flops / t / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"torch SDPA bf16 + attn_mask bias, first {q_rows} queries of segment 0 x all {L} keys x 16 heads,"
+                      f" median of 3 ({t:.2f} s each)"}
+
+
+def cpu_baseline_merge(mw):
+    import torch
+    import oracle
+
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    tokens = mw["tokens"][0].cpu()
+    conf = mw["conf"].cpu()
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        mask = oracle.select_lowest_confidence(conf, 1, 3, 3, mw["ratio"])
+        jag, rev = oracle.token_merge_2d(tokens, 5, 3, 3, 37, 37, mask, allow_remainder=True)
+        times.append(time.perf_counter() - t0)
+    t_merge = sorted(times)[1]
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        oracle.token_split(jag, rev, (1, mw["frames"], mw["N"], mw["C"]))
+        times.append(time.perf_counter() - t0)
+    t_split = sorted(times)[1]
+    return {"merge_GBs": round(mw["merge_bytes"] / t_merge / 1e9, 3), "unmerge_GBs": round(mw["split_bytes"] / t_split / 1e9, 3),
+            "cores": threads, "kind": "port",
+            "sample": f"oracle select+merge ({t_merge * 1e3:.0f} ms) and split ({t_split * 1e3:.0f} ms) of the full C2 "
+                      "workload on the CPU in bf16, median of 3"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
+              "multi-GPU sharding is a design note, not code. Re-run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from come_amd import _lib
+
+    _lib.load()                                                  # fails loudly when the HIP library is missing
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    if args.only:
+        if args.only == "attn":
+            w, wall, ev_ms = bench_attention(args.steps, args.warmup, device)
+            print(json.dumps({"only": "attn", "ms_per_call": ev_ms / args.steps,
+                              "tflops": w["flops"] / (ev_ms / args.steps * 1e-3) / 1e12}))
+        else:
+            mw = merge_workload(device)
+            for _ in range(8):
+                mw["merge_only"]()
+            fn = mw["merge_only"] if args.only == "merge" else mw["split_only"]
+            _, ms = time_loop(fn, args.steps, args.warmup)
+            nbytes = mw["merge_bytes"] if args.only == "merge" else mw["split_bytes"]
+            print(json.dumps({"only": args.only, "us_per_call": ms / args.steps * 1e3,
+                              "GBs": nbytes / (ms / args.steps * 1e-3) / 1e9}))
+        return
+
+    w, wall, ev_ms = bench_attention(args.steps, args.warmup, device)
+    ms_per_step = wall / args.steps * 1e3
+    value = w["flops"] / (wall / args.steps) / 1e12
+    kernel_tflops = w["flops"] / (ev_ms / args.steps * 1e-3) / 1e12
+
+    result = {
+        "metric": "biased-attn TFLOP/s",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "C3 biased varlen flash-attention fwd: 16 heads x 64, packed L = {25536, 21848} "
+                               "(32 frames 37x37 after 3x3 merge at r = 0.5 / 0.6), bias = log(count in {1,9}), "
+                               "scale 0.125, non-causal",
+                   "algorithmic_flops_per_step": w["flops"]},
+        "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(kernel_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "kernel": "attn_fwd_kernel<bf16>", "ms_per_launch": round(ev_ms / args.steps, 4)},
+    }
+    mw = None
+    if not args.no_other:
+        mw, other = bench_merge_unmerge(device)
+        result["other"] = other
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline_attention(w)
+        if mw is not None:
+            result["other"]["cpu_baseline"] = cpu_baseline_merge(mw)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
