@@ -20,7 +20,9 @@ OBJ_DIR = os.path.join(HERE, "build")
 SOURCES = ["abi.hip", "merge_kernels.hip", "select_kernels.hip", "attn_fwd.hip"]
 
 # Packed-FP32 VALU forms are switched off for all device code.
-DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                # MFMA accumulators in ordinary VGPRs: no v_accvgpr_read/write copies around the softmax
+                "-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 COMMON_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", "-Wall",
                 "-Wno-unused-function"] + DEVICE_FLAGS
 

@@ -23,6 +23,8 @@
 //   segment get t_hi = -inf, which makes their scores -inf and their probabilities 0.
 #include "come_common.h"
 
+#include <cstdlib>
+
 namespace come {
 namespace {
 
@@ -338,8 +340,8 @@ extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v,
                      (reinterpret_cast<uintptr_t>(v) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0,
                  COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: q/k/v must be 16-byte aligned, out 8-byte aligned");
 
-    constexpr int QT = 2;
-    constexpr int kBlockM = 128 * QT;
+    static const int QT = getenv("COME_ATTN_QT") ? atoi(getenv("COME_ATTN_QT")) : 2;
+    const int kBlockM = 128 * QT;
     AttnArgs a{};
     a.q = static_cast<const uint16_t *>(q);
     a.k = static_cast<const uint16_t *>(k);
@@ -362,10 +364,12 @@ extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v,
     COME_REQUIRE(n_wg < (1ll << 31), COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: grid too large");
     const dim3 grid(static_cast<unsigned>(n_wg)), block(kThreads);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == COME_BF16)
-        hipLaunchKernelGGL((attn_fwd_kernel<COME_BF16, QT>), grid, block, 0, s, a);
-    else
-        hipLaunchKernelGGL((attn_fwd_kernel<COME_F16, QT>), grid, block, 0, s, a);
+    if (dtype == COME_BF16) {
+        if (QT == 1) hipLaunchKernelGGL((attn_fwd_kernel<COME_BF16, 1>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((attn_fwd_kernel<COME_BF16, 2>), grid, block, 0, s, a);
+    } else {
+        hipLaunchKernelGGL((attn_fwd_kernel<COME_F16, 2>), grid, block, 0, s, a);
+    }
     COME_CHECK_LAUNCH("come_attn_varlen_fwd");
     return COME_OK;
 }

@@ -56,9 +56,14 @@ template <> struct Vec16<COME_F32> {
     __device__ static inline void store1(void *p, int64_t i, float v) { static_cast<float *>(p)[i] = v; }
 };
 
+typedef float come_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 come_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 come_f16x2 __attribute__((ext_vector_type(2)));
+
+// round-to-nearest-even of two floats into one packed word (one v_cvt_pk_bf16_f32)
 __device__ inline uint32_t pack2_bf16(float lo, float hi) {
-    __hip_bfloat162 r = __float22bfloat162_rn(make_float2(lo, hi));
-    return *reinterpret_cast<uint32_t *>(&r);
+    const come_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, come_bf16x2));
 }
 
 template <> struct Vec16<COME_BF16> {
@@ -85,8 +90,8 @@ template <> struct Vec16<COME_BF16> {
 };
 
 __device__ inline uint32_t pack2_f16(float lo, float hi) {
-    __half2 r = __floats2half2_rn(lo, hi);
-    return *reinterpret_cast<uint32_t *>(&r);
+    const come_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, come_f16x2));
 }
 
 template <> struct Vec16<COME_F16> {
