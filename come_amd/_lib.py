@@ -13,7 +13,8 @@ import threading
 import torch  # noqa: F401  (imported first so the process binds one HIP runtime, torch's)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libcome_hip.so")
+# COME_HIP_LIBRARY points at an alternative build of the same library (e.g. an experimental variant)
+LIB_PATH = os.environ.get("COME_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libcome_hip.so")
 
 COME_F32, COME_F16, COME_BF16 = 0, 1, 2
 
