@@ -40,6 +40,7 @@ constexpr int kBlockN = 64;          // keys per tile
 constexpr int kKPitch = 88;          // elements per K' row in LDS (64 + 16 bias/zero + 8 pad): 176 B, odd multiple of 16 B
 constexpr int kVPitch = 96;          // elements per V row in LDS: 192 B = 48 banks, 4 rows tile the 64 banks
 constexpr int kThreads = 256;
+constexpr int kBiasPitch = 24;       // elements per key of the bias / ones block (48 B: conflict-free 16-byte reads)
 
 struct AttnArgs {
     const uint16_t *q, *k, *v;
@@ -312,26 +313,44 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnArgs a) {
 
 
 // -------------------------------------------------------------------------------------
-// Software-pipelined variant: kBlockM = 256 queries per workgroup, two query tiles per
-// wavefront that alternate roles.  While the vector ALU runs the softmax of one query
-// tile, the matrix pipe runs the score MFMAs (next key tile) and the P V MFMAs (current
-// key tile) of the other one:
+// Software-pipelined kernel: kBlockM = 256 queries per workgroup, two query tiles per
+// wavefront that alternate roles.  While the vector ALU turns the scores of one query tile
+// into probabilities, the matrix pipe runs the score MFMAs (next key tile) and the P V MFMAs
+// (current key tile) of the other one:
 //
-//   slot a(j): VALU softmax(S0(j)) -> P0      MFMA S1(j) = K'(j) Q1'^T ; O1 += V(j-1)^T P1(j-1)
-//   slot b(j): VALU softmax(S1(j)) -> P1      MFMA S0(j+1) = K'(j+1) Q0'^T ; O0 += V(j)^T P0(j)
+//   slot a(j): VALU P0 = exp2(S0(j))      MFMA S1(j) = K'(j) Q1'^T ; O1 += V(j-1)^T P1(j-1)
+//   slot b(j): VALU P1 = exp2(S1(j))      MFMA S0(j+1) = K'(j+1) Q0'^T ; O0 += V(j)^T P0(j)
 //
-// K' tiles j, j+1 and V tiles j-1, j are live in one iteration, so LDS holds three tiles
-// of each and one barrier per iteration suffices.
+// K' tiles j, j+1 and V tiles j-1, j are live in one iteration, so LDS holds three tiles of each
+// and one barrier per iteration suffices.
+//
+// Scores leave the MFMA already in the form the exponential needs:
+//   S'' = (c q) . k + bias log2(e) - m,      c = softmax_scale log2(e)
+// Q is multiplied by c once (and rounded back to 16 bit); bias log2(e) and the reference point m of
+// the row ride through the fifth k-step as exact three-term 16-bit splits (K' carries the bias terms
+// and ones, Q' carries ones and the terms of -m).  m is the row maximum of the first key tile and is
+// moved only when a tile's row sum leaves a safe range (probabilities are then rescaled exactly as
+// in the usual online softmax); softmax is invariant to the choice of m, and fp32 / 16-bit floats
+// keep full relative precision for probabilities above 1.  The steady state therefore spends one
+// exp2, half a pack and half a dot per score on the vector ALU and nothing else.
 // -------------------------------------------------------------------------------------
 constexpr int kStages = 3;
+constexpr float kSumLimit = 16777216.f;      // 2^24: a tile row sum above this moves the reference point
 
 template <int DT>
 __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs a) {
     using E = Elem<DT>;
     constexpr int kBlockM = 256;
-    __shared__ __attribute__((aligned(16))) uint16_t lds_k[kStages][kBlockN * kKPitch];
-    __shared__ __attribute__((aligned(16))) uint16_t lds_v[kStages][kBlockN * kVPitch];
+    // K and V tiles: 64 rows of 128 bytes, unpadded, filled by direct global->LDS loads (a wavefront's
+    // load lands as 1 KiB in lane order); bank conflicts are avoided by permuting the 16-byte chunks
+    // inside a row: K chunk c of row r sits at slot c ^ ((r >> 1) & 7), V chunk c at c ^ (((r >> 1) & 1) << 2).
+    // lds_b: per key 48 bytes, [bias terms and ones (16 B) | zeros (16 B) | pad], the fifth k-step of K'.
+    __shared__ __attribute__((aligned(1024))) uint16_t lds_k[kStages][kBlockN * kHeadDim];
+    __shared__ __attribute__((aligned(1024))) uint16_t lds_v[kStages][kBlockN * kHeadDim];
+    __shared__ __attribute__((aligned(16))) uint16_t lds_b[kStages][kBlockN * kBiasPitch];
 
+    // consecutive query blocks of one (segment, head) run on the same XCD (workgroup i is
+    // dispatched to XCD i % 8) and share K/V in its L2
     const int n_wg = gridDim.x;
     int wid = blockIdx.x;
     const int per_xcd = n_wg >> 3;
@@ -350,97 +369,127 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
     const int wave = tid >> 6;
     const int h = lane >> 5;
     const int r = lane & 31;
+    constexpr float kLog2e = 1.4426950408889634f;
 
+    // ---- Q fragments (B operand: n = query r, k = head-dim 16 ks + 8 h ..), scaled by c
     u32x4 qf[2][4];
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
         const int row = q0 + (wave * 2 + qt) * 32 + r;
         const uint16_t *qp = a.q + static_cast<int64_t>(seq_start + min(row, L - 1)) * a.q_rs + head * a.q_hs + 8 * h;
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) qf[qt][ks] = *reinterpret_cast<const u32x4 *>(qp + 16 * ks);
+        for (int ks = 0; ks < 4; ++ks) {
+            const u32x4 raw = *reinterpret_cast<const u32x4 *>(qp + 16 * ks);
+#pragma unroll
+            for (int w = 0; w < 4; ++w)
+                qf[qt][ks][w] = E::pack2(E::to_f32(static_cast<uint16_t>(raw[w] & 0xffffu)) * a.scale_log2,
+                                         E::to_f32(static_cast<uint16_t>(raw[w] >> 16)) * a.scale_log2);
+        }
     }
-    const u32x4 q_ext = h == 0 ? u32x4{E::kOne | (E::kOne << 16), E::kOne, 0u, 0u} : zero4();
+    // fifth k-step of Q' (lower half-wave only): [1 1 1 | -m split in three | 0 0]
+    u32x4 q_ext[2];
+    q_ext[0] = h == 0 ? u32x4{E::kOne | (E::kOne << 16), E::kOne, 0u, 0u} : zero4();
+    q_ext[1] = q_ext[0];
 
-    const int sc = tid & 7;
-    const int sr = tid >> 3;
-    const uint16_t *k_base = a.k + static_cast<int64_t>(seq_start) * a.k_rs + head * a.k_hs + sc * 8;
-    const uint16_t *v_base = a.v + static_cast<int64_t>(seq_start) * a.v_rs + head * a.v_hs + sc * 8;
-    const uint16_t *b_base = a.bias ? a.bias + seq_start : nullptr;
-
-    // Global -> register staging.  Loads are unconditional: a key index beyond the segment is clamped to
-    // its last key (finite data); such keys get a bias term of -inf at commit time, so their
+    // ---- global -> LDS staging.  Wavefront w fills rows 16 w .. 16 w + 15 of a tile with two direct
+    // loads; lane l of load i brings row 8 (2 w + i) + l / 8, slot l % 8.  A key index beyond the segment
+    // is redirected to its last key (finite data); such keys get a bias term of -inf, so their
     // probabilities are exactly 0 and neither their K nor their V row can reach the output.
-    u32x4 k_stage[2], v_stage[2];
-    uint16_t b_raw = 0;
-    int b_key = 0;
-    // per-thread row pointers of key tile 0; a tile step is a wave-uniform offset
-    const uint16_t *k_row[2], *v_row[2];
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const char *k_seg = reinterpret_cast<const char *>(a.k + static_cast<int64_t>(seq_start) * a.k_rs + head * a.k_hs);
+    const char *v_seg = reinterpret_cast<const char *>(a.v + static_cast<int64_t>(seq_start) * a.v_rs + head * a.v_hs);
+    const uint16_t *b_base = a.bias ? a.bias + seq_start : nullptr;
+    const uint32_t k_rs_b = static_cast<uint32_t>(a.k_rs) * 2u, v_rs_b = static_cast<uint32_t>(a.v_rs) * 2u;
+    uint32_t k_goff[2], v_goff[2], k_chunk[2], v_chunk[2];
+    int st_row[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        k_row[i] = k_base + static_cast<int64_t>(sr + 32 * i) * a.k_rs;
-        v_row[i] = v_base + static_cast<int64_t>(sr + 32 * i) * a.v_rs;
+        st_row[i] = 8 * (2 * wave + i) + (lane >> 3);
+        k_chunk[i] = static_cast<uint32_t>((lane & 7) ^ ((st_row[i] >> 1) & 7)) * 16u;
+        v_chunk[i] = static_cast<uint32_t>((lane & 7) ^ (((st_row[i] >> 1) & 1) << 2)) * 16u;
+        k_goff[i] = static_cast<uint32_t>(st_row[i]) * k_rs_b + k_chunk[i];
+        v_goff[i] = static_cast<uint32_t>(st_row[i]) * v_rs_b + v_chunk[i];
     }
-    const uint16_t *k_last = k_base + static_cast<int64_t>(L - 1) * a.k_rs;
-    const uint16_t *v_last = v_base + static_cast<int64_t>(L - 1) * a.v_rs;
-    const int64_t k_tile_step = static_cast<int64_t>(kBlockN) * a.k_rs;
-    const int64_t v_tile_step = static_cast<int64_t>(kBlockN) * a.v_rs;
-    auto fetch_k = [&](int tile) {
+    const uint32_t k_last = static_cast<uint32_t>(L - 1) * k_rs_b, v_last = static_cast<uint32_t>(L - 1) * v_rs_b;
+    const uint32_t k_tile_step = static_cast<uint32_t>(kBlockN) * k_rs_b, v_tile_step = static_cast<uint32_t>(kBlockN) * v_rs_b;
+
+    uint16_t b_raw = 0;
+    int b_key = 0;
+    auto stage_k = [&](int tile, int buf) {
         const int n0 = tile * kBlockN;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const uint16_t *p = n0 + sr + 32 * i < L ? k_row[i] + tile * k_tile_step : k_last;
-            k_stage[i] = *reinterpret_cast<const u32x4 *>(p);
+            const uint32_t off = n0 + st_row[i] < L ? static_cast<uint32_t>(tile) * k_tile_step + k_goff[i] : k_last + k_chunk[i];
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(k_seg + off),
+                                             (__attribute__((address_space(3))) void *)(&lds_k[buf][(2 * wave_u + i) * 512]),
+                                             16, 0, 0);
         }
         if (tid < kBlockN) {
             b_key = n0 + tid;
             if (b_base) b_raw = b_base[min(b_key, L - 1)];
         }
     };
-    auto fetch_v = [&](int tile) {
+    auto stage_v = [&](int tile, int buf) {
         const int n0 = tile * kBlockN;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const uint16_t *p = n0 + sr + 32 * i < L ? v_row[i] + tile * v_tile_step : v_last;
-            v_stage[i] = *reinterpret_cast<const u32x4 *>(p);
+            const uint32_t off = n0 + st_row[i] < L ? static_cast<uint32_t>(tile) * v_tile_step + v_goff[i] : v_last + v_chunk[i];
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(v_seg + off),
+                                             (__attribute__((address_space(3))) void *)(&lds_v[buf][(2 * wave_u + i) * 512]),
+                                             16, 0, 0);
         }
     };
-    auto commit_k = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-            *reinterpret_cast<u32x4 *>(&lds_k[buf][(sr + 32 * i) * kKPitch + sc * 8]) = k_stage[i];
+    // exact three-term 16-bit split of an fp32 value (an infinite value stays one term)
+    auto split3 = [&](float t, uint32_t &t_hi, uint32_t &t_mid, uint32_t &t_lo) {
+        t_hi = E::from_f32(t);
+        t_mid = 0;
+        t_lo = 0;
+        const float hi_f = E::to_f32(static_cast<uint16_t>(t_hi));
+        if (fabsf(hi_f) != INFINITY) {
+            const float r1 = t - hi_f;
+            t_mid = E::from_f32(r1);
+            t_lo = E::from_f32(r1 - E::to_f32(static_cast<uint16_t>(t_mid)));
+        }
+    };
+    auto commit_bias = [&](int buf) {
         if (tid < kBlockN) {
-            // t = bias / scale split exactly into three 16-bit terms; -inf beyond the segment
-            const float t = b_base ? E::to_f32(b_raw) * a.inv_scale : 0.f;
-            uint32_t t_hi = E::from_f32(t), t_mid = 0, t_lo = 0;
-            const float hi_f = E::to_f32(static_cast<uint16_t>(t_hi));
-            if (fabsf(hi_f) != INFINITY) {
-                const float r1 = t - hi_f;
-                t_mid = E::from_f32(r1);
-                t_lo = E::from_f32(r1 - E::to_f32(static_cast<uint16_t>(t_mid)));
-            }
+            // [bias log2(e) in three terms | 1 1 1 | 0 0] then 16 bytes of zeros; -inf beyond the segment
+            uint32_t t_hi, t_mid, t_lo;
+            split3(b_base ? E::to_f32(b_raw) * kLog2e : 0.f, t_hi, t_mid, t_lo);
             if (b_key >= L) {
                 t_hi = E::kNegInf;
                 t_mid = 0;
                 t_lo = 0;
             }
-            *reinterpret_cast<u32x4 *>(&lds_k[buf][tid * kKPitch + 64]) = u32x4{t_hi | (t_mid << 16), t_lo, 0u, 0u};
-            *reinterpret_cast<u32x4 *>(&lds_k[buf][tid * kKPitch + 72]) = zero4();
+            *reinterpret_cast<u32x4 *>(&lds_b[buf][tid * kBiasPitch]) =
+                u32x4{t_hi | (t_mid << 16), t_lo | (E::kOne << 16), E::kOne | (E::kOne << 16), 0u};
+            *reinterpret_cast<u32x4 *>(&lds_b[buf][tid * kBiasPitch + 8]) = zero4();
         }
     };
-    auto commit_v = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-            *reinterpret_cast<u32x4 *>(&lds_v[buf][(sr + 32 * i) * kVPitch + sc * 8]) = v_stage[i];
+    // all direct loads of this wavefront have landed, then the workgroup meets
+    auto staged_barrier = [&]() {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
     };
 
-    const int k_off = r * kKPitch + 8 * h;
-    const int v_off = (4 * h + ((lane & 15) >> 2)) * kVPitch + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    // LDS read offsets (in elements) of this lane
+    int k_rd[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) k_rd[ks] = r * kHeadDim + (((2 * ks + h) ^ ((r >> 1) & 7)) << 3);
+    const int b_rd = r * kBiasPitch + 8 * h;
+    const int i16 = lane & 15;
+    int v_rd[2];
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+        v_rd[dt] = (4 * h + (i16 >> 2)) * kHeadDim +
+                   (((4 * dt + 2 * ((lane >> 4) & 1) + ((i16 & 3) >> 1)) ^ (((i16 >> 3) & 1) << 2)) << 3) + 4 * (i16 & 1);
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-    f32x16 s_acc[2][2];          // scores of the two query tiles (two 32-key halves each)
+    f32x16 s_acc[2][2];          // S'' of the two query tiles (two 32-key halves each)
     f32x16 o_acc[2][2];
     u32x4 p_frag[2][4];
-    float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
+    float m_run[2] = {0.f, 0.f};  // reference point of the row, log2 units
+    float l_run[2] = {0.f, 0.f};  // per-lane partial row sum
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
         o_acc[qt][0] = zero16;
@@ -449,111 +498,55 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
         for (int u = 0; u < 4; ++u) p_frag[qt][u] = zero4();
     }
 
-    // scores of query tile `qt` against the K' tile in `buf`
     auto score_mfma = [&](int qt, int buf) {
 #pragma unroll
         for (int ks = 0; ks < 5; ++ks) {
-#ifdef COME_EXP_NO_LDSREAD
-            const u32x4 kf0 = qf[qt ^ 1][ks & 3], kf1 = qf[qt ^ 1][(ks + 1) & 3];
-#else
-            const u32x4 kf0 = *reinterpret_cast<const u32x4 *>(&lds_k[buf][k_off + 16 * ks]);
-            const u32x4 kf1 = *reinterpret_cast<const u32x4 *>(&lds_k[buf][k_off + 32 * kKPitch + 16 * ks]);
-#endif
-            const u32x4 qb = ks < 4 ? qf[qt][ks < 4 ? ks : 0] : q_ext;
+            const uint16_t *kp = ks < 4 ? &lds_k[buf][k_rd[ks < 4 ? ks : 0]] : &lds_b[buf][b_rd];
+            const u32x4 kf0 = *reinterpret_cast<const u32x4 *>(kp);
+            const u32x4 kf1 = *reinterpret_cast<const u32x4 *>(kp + 32 * (ks < 4 ? kHeadDim : kBiasPitch));
+            const u32x4 qb = ks < 4 ? qf[qt][ks < 4 ? ks : 0] : q_ext[qt];
             s_acc[qt][0] = E::mfma(kf0, qb, ks == 0 ? zero16 : s_acc[qt][0]);
             s_acc[qt][1] = E::mfma(kf1, qb, ks == 0 ? zero16 : s_acc[qt][1]);
         }
     };
-    // O^T += V^T P^T of query tile `qt` with the V tile in `buf`
     auto pv_mfma = [&](int qt, int buf) {
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt) {
-                const uint16_t *vp = &lds_v[buf][v_off + (16 * u) * kVPitch + 32 * dt];
-#ifdef COME_EXP_NO_LDSREAD
-                (void)vp;
-                const u32x2 lo2 = {qf[qt][u][0], qf[qt][u][1]}, hi2 = {qf[qt][u][2], qf[qt][u][3]};
-#else
+                const uint16_t *vp = &lds_v[buf][v_rd[dt] + (16 * u) * kHeadDim];
                 const u32x2 lo2 = __builtin_bit_cast(u32x2, lds_read_tr(vp));
-                const u32x2 hi2 = __builtin_bit_cast(u32x2, lds_read_tr(vp + 8 * kVPitch));
-#endif
+                const u32x2 hi2 = __builtin_bit_cast(u32x2, lds_read_tr(vp + 8 * kHeadDim));
                 o_acc[qt][dt] = E::mfma(u32x4{lo2[0], lo2[1], hi2[0], hi2[1]}, p_frag[qt][u], o_acc[qt][dt]);
             }
         }
     };
-    // online softmax of query tile `qt`: S -> P (16-bit B operands), updates m, l; returns the O rescale factor
-    auto softmax = [&](int qt) -> float {
-        float mx0 = fmaxf(s_acc[qt][0][0], s_acc[qt][0][1]);
-        float mx1 = fmaxf(s_acc[qt][0][8], s_acc[qt][0][9]);
-        float mx2 = fmaxf(s_acc[qt][1][0], s_acc[qt][1][1]);
-        float mx3 = fmaxf(s_acc[qt][1][8], s_acc[qt][1][9]);
-#pragma unroll
-        for (int i = 2; i < 8; i += 2) {
-            mx0 = fmaxf(fmaxf(mx0, s_acc[qt][0][i]), s_acc[qt][0][i + 1]);
-            mx1 = fmaxf(fmaxf(mx1, s_acc[qt][0][8 + i]), s_acc[qt][0][9 + i]);
-            mx2 = fmaxf(fmaxf(mx2, s_acc[qt][1][i]), s_acc[qt][1][i + 1]);
-            mx3 = fmaxf(fmaxf(mx3, s_acc[qt][1][8 + i]), s_acc[qt][1][9 + i]);
-        }
-        float mx = fmaxf(fmaxf(mx0, mx1), fmaxf(mx2, mx3));
-        mx = max_across_halves(mx);
-        const float m_new = fmaxf(m_run[qt], mx);
-        const float m_use = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_use) * a.scale_log2);
-        const float mc = m_use * a.scale_log2;
-        float sum = 0.f;
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                u32x4 f;
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-#ifdef COME_EXP_NO_SOFTMAX
-                    const float p0 = s_acc[qt][mt][8 * t + 2 * w], p1 = s_acc[qt][mt][8 * t + 2 * w + 1];
-                    f[w] = __float_as_uint(p0) ^ __float_as_uint(p1);
-#else
-                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[qt][mt][8 * t + 2 * w], a.scale_log2, -mc));
-                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[qt][mt][8 * t + 2 * w + 1], a.scale_log2, -mc));
-                    f[w] = E::pack2(p0, p1);
-                    sum = E::dot2_ones(f[w], sum);
-#endif
-                }
-                p_frag[qt][2 * mt + t] = f;
-            }
-        }
-        l_run[qt] = l_run[qt] * alpha + sum;
-        m_run[qt] = m_new;
-        // ties the rescale decision to the end of the softmax, so the branch that follows cannot be
-        // hoisted into the middle of it and the whole slot stays one scheduling region
-        float alpha_late = alpha;
-        asm volatile("" : "+v"(alpha_late) : "v"(sum), "v"(p_frag[qt][3][3]));
-        return alpha_late;
-    };
+
     // One slot in explicit issue order.  The matrix pipe works on query tile Y: 10 score MFMAs against
-    // the K' tile in `kbuf` (S[Y] is rebuilt), then 8 P V MFMAs with the V tile in `vbuf` (P[Y] from
-    // the previous slot).  The vector ALU runs the softmax of query tile X in between: MFMA i is
-    // followed by a chunk of softmax work, and the LDS reads of MFMA i + 2 are requested before it,
-    // so an in-order wavefront always has independent vector work behind every MFMA.
-    // sched_barrier keeps the compiler from regrouping the chunks.
+    // the K' tile in `kbuf` (S[Y] is rebuilt), then 8 P V MFMAs with the V tile in `vbuf` (P[Y] from the
+    // previous slot).  The vector ALU turns S[X] into P[X] in between: every MFMA is followed by a
+    // chunk of vector work, and the LDS reads of MFMA i + 2 are requested before it, so an in-order
+    // wavefront always has independent vector work behind each MFMA.  sched_barrier keeps the compiler
+    // from regrouping the chunks.  Returns the tile row sum of this lane.
     auto slot = [&](int X, int Y, int kbuf, int vbuf) -> float {
         u32x4 frag[18];
         auto request = [&](int i) {
             if (i < 10) {
                 const int ks = i >> 1, mt = i & 1;
-                frag[i] = *reinterpret_cast<const u32x4 *>(&lds_k[kbuf][k_off + 32 * mt * kKPitch + 16 * ks]);
+                frag[i] = ks < 4 ? *reinterpret_cast<const u32x4 *>(&lds_k[kbuf][k_rd[ks < 4 ? ks : 0] + 32 * mt * kHeadDim])
+                                 : *reinterpret_cast<const u32x4 *>(&lds_b[kbuf][b_rd + 32 * mt * kBiasPitch]);
             } else if (i < 18) {
                 const int u = (i - 10) >> 1, dt = (i - 10) & 1;
-                const uint16_t *vp = &lds_v[vbuf][v_off + (16 * u) * kVPitch + 32 * dt];
+                const uint16_t *vp = &lds_v[vbuf][v_rd[dt] + (16 * u) * kHeadDim];
                 const u32x2 lo2 = __builtin_bit_cast(u32x2, lds_read_tr(vp));
-                const u32x2 hi2 = __builtin_bit_cast(u32x2, lds_read_tr(vp + 8 * kVPitch));
+                const u32x2 hi2 = __builtin_bit_cast(u32x2, lds_read_tr(vp + 8 * kHeadDim));
                 frag[i] = u32x4{lo2[0], lo2[1], hi2[0], hi2[1]};
             }
         };
         auto issue = [&](int i) {
             if (i < 10) {
                 const int ks = i >> 1, mt = i & 1;
-                const u32x4 qb = ks < 4 ? qf[Y][ks < 4 ? ks : 0] : q_ext;
+                const u32x4 qb = ks < 4 ? qf[Y][ks < 4 ? ks : 0] : q_ext[Y];
                 s_acc[Y][mt] = E::mfma(frag[i], qb, ks == 0 ? zero16 : s_acc[Y][mt]);
             } else {
                 const int u = (i - 10) >> 1, dt = (i - 10) & 1;
@@ -562,84 +555,84 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
         };
         request(0);
         request(1);
-        // -- chunk 0: four partial maxima
-        issue(0);
-        request(2);
-        float mx0 = fmaxf(s_acc[X][0][0], s_acc[X][0][1]);
-        float mx1 = fmaxf(s_acc[X][0][8], s_acc[X][0][9]);
-        float mx2 = fmaxf(s_acc[X][1][0], s_acc[X][1][1]);
-        float mx3 = fmaxf(s_acc[X][1][8], s_acc[X][1][9]);
-#pragma unroll
-        for (int e = 2; e < 8; e += 2) {
-            mx0 = fmaxf(fmaxf(mx0, s_acc[X][0][e]), s_acc[X][0][e + 1]);
-            mx1 = fmaxf(fmaxf(mx1, s_acc[X][0][8 + e]), s_acc[X][0][9 + e]);
-            mx2 = fmaxf(fmaxf(mx2, s_acc[X][1][e]), s_acc[X][1][e + 1]);
-            mx3 = fmaxf(fmaxf(mx3, s_acc[X][1][8 + e]), s_acc[X][1][9 + e]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // -- chunk 1: row max across the two half-waves, new running max, rescale factor
-        issue(1);
-        request(3);
-        float mx = fmaxf(fmaxf(mx0, mx1), fmaxf(mx2, mx3));
-        mx = max_across_halves(mx);
-        const float m_new = fmaxf(m_run[X], mx);
-        const float m_use = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f((m_run[X] - m_use) * a.scale_log2);
-        const float mc = m_use * a.scale_log2;
         float sum = 0.f;
-        __builtin_amdgcn_sched_barrier(0);
-        // -- chunks 2..17: one pair of probabilities each
+        float p0 = 0.f, p1 = 0.f;
 #pragma unroll
         for (int c = 0; c < 16; ++c) {
-            issue(2 + c);
-            request(4 + c);
-            const int mt = c >> 3, t = (c >> 2) & 1, w = c & 3;
-            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[X][mt][8 * t + 2 * w], a.scale_log2, -mc));
-            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[X][mt][8 * t + 2 * w + 1], a.scale_log2, -mc));
-            const uint32_t pw = E::pack2(p0, p1);
-            p_frag[X][2 * mt + t][w] = pw;
-            sum = E::dot2_ones(pw, sum);
+            issue(c);
+            request(c + 2);
+            if (c > 0) {                    // pack and add the pair whose exponentials were issued one chunk ago
+                const int pc = c - 1;
+                const uint32_t pw = E::pack2(p0, p1);
+                p_frag[X][pc >> 2][pc & 3] = pw;
+                sum = E::dot2_ones(pw, sum);
+            }
+            p0 = __builtin_amdgcn_exp2f(s_acc[X][c >> 3][2 * (c & 7)]);
+            p1 = __builtin_amdgcn_exp2f(s_acc[X][c >> 3][2 * (c & 7) + 1]);
             __builtin_amdgcn_sched_barrier(0);
         }
+        issue(16);
+        {
+            const uint32_t pw = E::pack2(p0, p1);
+            p_frag[X][3][3] = pw;
+            sum = E::dot2_ones(pw, sum);
+        }
+        issue(17);
+        // the decision that follows the slot is tied to its end, so that the branch cannot be moved
+        // above the probability chunks
+        float sum_late = sum;
+        asm volatile("" : "+v"(sum_late) : "v"(p_frag[X][3][3]));
+        return sum_late;
+    };
+
+    // Exact path of query tile X: move the reference point to the row maximum of this tile and redo its
+    // probabilities.  The scores are rebuilt from the K' tile (still in LDS) rather than kept alive
+    // through the slot, which would cost 32 registers in the steady state for a path that is almost
+    // never taken.
+    auto recentre = [&](int X, int kbuf) {
+        score_mfma(X, kbuf);
+        float mx = s_acc[X][0][0];
+#pragma unroll
+        for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s_acc[X][0][e]);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[X][1][e]);
+        mx = max_across_halves(mx);
+        const float delta = mx == -INFINITY ? 0.f : mx;          // every key masked so far: stay put
+        float sum = 0.f;
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            const float p0 = __builtin_amdgcn_exp2f(s_acc[X][c >> 3][2 * (c & 7)] - delta);
+            const float p1 = __builtin_amdgcn_exp2f(s_acc[X][c >> 3][2 * (c & 7) + 1] - delta);
+            const uint32_t pw = E::pack2(p0, p1);
+            p_frag[X][c >> 2][c & 3] = pw;
+            sum = E::dot2_ones(pw, sum);
+            __builtin_amdgcn_sched_barrier(0);      // rare path: keep it serial and small in registers
+        }
+        const float alpha = __builtin_amdgcn_exp2f(fminf(-delta, 126.f));   // what was accumulated so far shrinks
+        // in-place multiplies: written as asm so that the accumulator tuples keep their registers across
+        // this rarely taken branch (a plain multiply makes the allocator copy both 16-register tuples)
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                float t = o_acc[X][dt][e];
+                asm volatile("v_mul_f32 %0, %1, %0" : "+v"(t) : "v"(alpha));
+                o_acc[X][dt][e] = t;
+            }
         l_run[X] = l_run[X] * alpha + sum;
-        m_run[X] = m_new;
-        // the rescale decision is tied to the end of the slot so that the branch which follows cannot be
-        // moved above the probability chunks
-        float alpha_late = alpha;
-        asm volatile("" : "+v"(alpha_late) : "v"(sum), "v"(p_frag[X][3][3]));
-        return alpha_late;
-    };
-
-    auto rescale = [&](int qt, float alpha) {
-        if (__any(alpha != 1.0f)) {
-#pragma unroll
-            for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) o_acc[qt][dt][i] *= alpha;
+        m_run[X] += delta;
+        uint32_t n_hi, n_mid, n_lo;
+        split3(-m_run[X], n_hi, n_mid, n_lo);
+        if (h == 0) {
+            q_ext[X][1] = E::kOne | (n_hi << 16);
+            q_ext[X][2] = n_mid | (n_lo << 16);
         }
     };
-
-    // asks the scheduler to issue one slot as: LDS reads ahead, then 18 x {1 MFMA, LDS reads, ~7 VALU}
-    auto interleave_hint = [&]() {
-        // operand fragments are requested two MFMAs ahead of their use: 10 score MFMAs take one
-        // ds_read_b128 each, 8 P V MFMAs two transposing reads each
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x402, 7, 0);
-        }
-#pragma unroll
-        for (int i = 8; i < 16; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x402, 7, 0);
-        }
-#pragma unroll
-        for (int i = 16; i < 18; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x402, 7, 0);
+    auto finish_slot = [&](int X, int kbuf, float sum, bool force) {
+        if (force || __any(!(sum <= kSumLimit))) {
+            recentre(X, kbuf);
+        } else {
+            l_run[X] += sum;
         }
     };
 
@@ -647,43 +640,35 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
     const int n_tiles = (L + kBlockN - 1) / kBlockN;
     {   // V stage 2 stands in for "tile -1": zeros (P1 is zero there as well)
         u32x4 *z = reinterpret_cast<u32x4 *>(&lds_v[2][0]);
-        for (int i = tid; i < kBlockN * kVPitch / 8; i += kThreads) z[i] = zero4();
+        for (int i = tid; i < kBlockN * kHeadDim / 8; i += kThreads) z[i] = zero4();
     }
-    fetch_k(0);
-    fetch_v(0);
-    commit_k(0);
-    commit_v(0);
-    fetch_k(1);
-    commit_k(1);
-    __syncthreads();
+    stage_k(0, 0);
+    stage_v(0, 0);
+    commit_bias(0);
+    stage_k(1, 1);
+    commit_bias(1);
+    staged_barrier();
     score_mfma(0, 0);
 
     int kb = 0;                  // stage of K'(j) and V(j); K'(j+1) is in kb + 1, V(j-1) in kb + 2 (mod 3)
     for (int j = 0; j < n_tiles; ++j) {
         const int kb1 = kb == 2 ? 0 : kb + 1;
         const int kb2 = kb1 == 2 ? 0 : kb1 + 1;
-#ifndef COME_EXP_NO_STAGE
-        fetch_k(j + 2);
-        fetch_v(j + 1);
-#endif
+        stage_k(j + 2, kb2);           // K'(j+2) replaces K'(j-1), V(j+1) replaces V(j-2): both idle since the
+        stage_v(j + 1, kb1);           // last barrier; the data is first read after the next one
 
-        const float alpha0 = slot(0, 1, kb, kb2);      // slot a
-        rescale(0, alpha0);
-        const float alpha1 = slot(1, 0, kb1, kb);      // slot b
-        rescale(1, alpha1);
+        const float sum0 = slot(0, 1, kb, kb2);        // slot a
+        finish_slot(0, kb, sum0, j == 0);
+        const float sum1 = slot(1, 0, kb1, kb);        // slot b
+        finish_slot(1, kb, sum1, j == 0);
 
-#ifndef COME_EXP_NO_STAGE
-        commit_k(kb2);
-        commit_v(kb1);
-#endif
-#ifndef COME_EXP_NO_BARRIER
-        __syncthreads();
-#endif
+        commit_bias(kb2);
+        staged_barrier();
         kb = kb1;
     }
-    // V(n-1) now sits in stage kb + 2 (mod 3)
-    pv_mfma(1, kb == 0 ? 2 : kb - 1);
+    pv_mfma(1, kb == 0 ? 2 : kb - 1);      // V(n-1)
 
+    // ---- epilogue: normalise, write O (and LSE)
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
         const float l_tot = sum_across_halves(l_run[qt]);
@@ -701,7 +686,8 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
                     *reinterpret_cast<u32x2 *>(op + 32 * dt + 8 * g) = w;
                 }
             if (h == 0 && a.lse)
-                a.lse[static_cast<int64_t>(head) * a.total + seq_start + row] = m_run[qt] * a.scale + __logf(l_tot);
+                a.lse[static_cast<int64_t>(head) * a.total + seq_start + row] =
+                    (m_run[qt] + __log2f(l_tot)) * 0.6931471805599453f;
         }
     }
 }
