@@ -321,8 +321,8 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnArgs a) {
 //   slot a(j): VALU P0 = exp2(S0(j))      MFMA S1(j) = K'(j) Q1'^T ; O1 += V(j-1)^T P1(j-1)
 //   slot b(j): VALU P1 = exp2(S1(j))      MFMA S0(j+1) = K'(j+1) Q0'^T ; O0 += V(j)^T P0(j)
 //
-// K' tiles j, j+1 and V tiles j-1, j are live in one iteration, so LDS holds three tiles of each
-// and one barrier per iteration suffices.
+// K' tiles j, j+1 and V tiles j-1, j are live in one iteration and the tiles of the next iteration
+// are in flight from global memory, so LDS holds four tiles of each; one barrier per iteration.
 //
 // Scores leave the MFMA already in the form the exponential needs:
 //   S'' = (c q) . k + bias log2(e) - m,      c = softmax_scale log2(e)
@@ -334,7 +334,22 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnArgs a) {
 // keep full relative precision for probabilities above 1.  The steady state therefore spends one
 // exp2, half a pack and half a dot per score on the vector ALU and nothing else.
 // -------------------------------------------------------------------------------------
-constexpr int kStages = 3;
+constexpr int kStages = 4;
+
+// Direct global -> LDS loads (lane l of the wavefront lands at lds_addr + 16 l, resp. + 4 l), written as
+// asm so that the compiler does not order them against LDS reads it cannot tell apart: completion is
+// awaited explicitly with s_waitcnt vmcnt before the barrier that publishes the tile.
+__device__ inline void dma_b128(const char *base, uint32_t lane_offset, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory");
+}
+__device__ inline void dma_b32(const char *base, uint32_t lane_offset, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                 :: "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory");
+}
+__device__ inline uint32_t lds_address(const void *p) {
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void *)(p)));
+}
 constexpr float kSumLimit = 16777216.f;      // 2^24: a tile row sum above this moves the reference point
 
 template <int DT>
@@ -348,6 +363,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
     __shared__ __attribute__((aligned(1024))) uint16_t lds_k[kStages][kBlockN * kHeadDim];
     __shared__ __attribute__((aligned(1024))) uint16_t lds_v[kStages][kBlockN * kHeadDim];
     __shared__ __attribute__((aligned(16))) uint16_t lds_b[kStages][kBlockN * kBiasPitch];
+    __shared__ __attribute__((aligned(256))) uint32_t lds_braw[kStages][kBlockN];   // raw bias words as loaded
 
     // consecutive query blocks of one (segment, head) run on the same XCD (workgroup i is
     // dispatched to XCD i % 8) and share K/V in its L2
@@ -398,7 +414,10 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const char *k_seg = reinterpret_cast<const char *>(a.k + static_cast<int64_t>(seq_start) * a.k_rs + head * a.k_hs);
     const char *v_seg = reinterpret_cast<const char *>(a.v + static_cast<int64_t>(seq_start) * a.v_rs + head * a.v_hs);
-    const uint16_t *b_base = a.bias ? a.bias + seq_start : nullptr;
+    // bias of the segment as bytes from a 4-byte aligned base: b_mis is the misalignment of its first key
+    const uintptr_t b_addr = reinterpret_cast<uintptr_t>(a.bias) + 2u * static_cast<uintptr_t>(seq_start);
+    const char *b_seg = a.bias ? reinterpret_cast<const char *>(b_addr & ~static_cast<uintptr_t>(3)) : nullptr;
+    const uint32_t b_mis = static_cast<uint32_t>(b_addr & 3);
     const uint32_t k_rs_b = static_cast<uint32_t>(a.k_rs) * 2u, v_rs_b = static_cast<uint32_t>(a.v_rs) * 2u;
     uint32_t k_goff[2], v_goff[2], k_chunk[2], v_chunk[2];
     int st_row[2];
@@ -413,20 +432,20 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
     const uint32_t k_last = static_cast<uint32_t>(L - 1) * k_rs_b, v_last = static_cast<uint32_t>(L - 1) * v_rs_b;
     const uint32_t k_tile_step = static_cast<uint32_t>(kBlockN) * k_rs_b, v_tile_step = static_cast<uint32_t>(kBlockN) * v_rs_b;
 
-    uint16_t b_raw = 0;
-    int b_key = 0;
     auto stage_k = [&](int tile, int buf) {
         const int n0 = tile * kBlockN;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const uint32_t off = n0 + st_row[i] < L ? static_cast<uint32_t>(tile) * k_tile_step + k_goff[i] : k_last + k_chunk[i];
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(k_seg + off),
-                                             (__attribute__((address_space(3))) void *)(&lds_k[buf][(2 * wave_u + i) * 512]),
-                                             16, 0, 0);
+            dma_b128(k_seg, off, lds_address(&lds_k[buf][(2 * wave_u + i) * 512]));
         }
-        if (tid < kBlockN) {
-            b_key = n0 + tid;
-            if (b_base) b_raw = b_base[min(b_key, L - 1)];
+    };
+    // raw bias of the 64 keys of a tile: wavefront 0 brings the aligned 32-bit word that holds each key's
+    // 16-bit bias; it is converted into the fifth k-step block one iteration later (commit_bias)
+    auto load_bias = [&](int tile, int buf) {
+        if (wave_u == 0 && b_seg) {
+            const uint32_t key = static_cast<uint32_t>(min(tile * kBlockN + lane, L - 1));
+            dma_b32(b_seg, ((b_mis + 2u * key) & ~3u), lds_address(&lds_braw[buf][0]));
         }
     };
     auto stage_v = [&](int tile, int buf) {
@@ -434,9 +453,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const uint32_t off = n0 + st_row[i] < L ? static_cast<uint32_t>(tile) * v_tile_step + v_goff[i] : v_last + v_chunk[i];
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(v_seg + off),
-                                             (__attribute__((address_space(3))) void *)(&lds_v[buf][(2 * wave_u + i) * 512]),
-                                             16, 0, 0);
+            dma_b128(v_seg, off, lds_address(&lds_v[buf][(2 * wave_u + i) * 512]));
         }
     };
     // exact three-term 16-bit split of an fp32 value (an infinite value stays one term)
@@ -451,24 +468,39 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
             t_lo = E::from_f32(r1 - E::to_f32(static_cast<uint16_t>(t_mid)));
         }
     };
-    auto commit_bias = [&](int buf) {
-        if (tid < kBlockN) {
+    auto commit_bias = [&](int tile, int buf) {
+        if (wave_u == 0) {
             // [bias log2(e) in three terms | 1 1 1 | 0 0] then 16 bytes of zeros; -inf beyond the segment
+            const int key = tile * kBlockN + lane;
+            float bias = 0.f;
+            if (b_seg) {
+                const uint32_t word = lds_braw[buf][lane];
+                const uint32_t at = b_mis + 2u * static_cast<uint32_t>(min(key, L - 1));
+                bias = E::to_f32(static_cast<uint16_t>((at & 2u) ? (word >> 16) : (word & 0xffffu)));
+            }
             uint32_t t_hi, t_mid, t_lo;
-            split3(b_base ? E::to_f32(b_raw) * kLog2e : 0.f, t_hi, t_mid, t_lo);
-            if (b_key >= L) {
+            split3(bias * kLog2e, t_hi, t_mid, t_lo);
+            if (key >= L) {
                 t_hi = E::kNegInf;
                 t_mid = 0;
                 t_lo = 0;
             }
-            *reinterpret_cast<u32x4 *>(&lds_b[buf][tid * kBiasPitch]) =
+            *reinterpret_cast<u32x4 *>(&lds_b[buf][lane * kBiasPitch]) =
                 u32x4{t_hi | (t_mid << 16), t_lo | (E::kOne << 16), E::kOne | (E::kOne << 16), 0u};
-            *reinterpret_cast<u32x4 *>(&lds_b[buf][tid * kBiasPitch + 8]) = zero4();
+            *reinterpret_cast<u32x4 *>(&lds_b[buf][lane * kBiasPitch + 8]) = zero4();
         }
     };
-    // all direct loads of this wavefront have landed, then the workgroup meets
-    auto staged_barrier = [&]() {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // the loads issued one iteration ago have landed (only the four direct loads of this iteration, plus
+    // the bias load in wavefront 0, may still be in flight), then the workgroup meets
+    auto staged_wait = [&]() {
+        if (wave_u == 0 && b_seg) {
+            asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        }
+    };
+    auto staged_barrier = [&](bool) {
+        staged_wait();
         __syncthreads();
     };
 
@@ -638,35 +670,47 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
 
     // ---- prologue
     const int n_tiles = (L + kBlockN - 1) / kBlockN;
-    {   // V stage 2 stands in for "tile -1": zeros (P1 is zero there as well)
-        u32x4 *z = reinterpret_cast<u32x4 *>(&lds_v[2][0]);
+    {   // the last V stage stands in for "tile -1": zeros (P1 is zero there as well)
+        u32x4 *z = reinterpret_cast<u32x4 *>(&lds_v[kStages - 1][0]);
         for (int i = tid; i < kBlockN * kHeadDim / 8; i += kThreads) z[i] = zero4();
     }
+    load_bias(0, 0);
+    load_bias(1, 1);
     stage_k(0, 0);
     stage_v(0, 0);
-    commit_bias(0);
     stage_k(1, 1);
-    commit_bias(1);
-    staged_barrier();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    commit_bias(0, 0);
+    commit_bias(1, 1);
+    load_bias(2, 2);                   // tiles of iteration 1 start their flight
+    stage_k(2, 2);
+    stage_v(1, 1);
+    staged_barrier(false);             // everything but this last group has landed
     score_mfma(0, 0);
 
-    int kb = 0;                  // stage of K'(j) and V(j); K'(j+1) is in kb + 1, V(j-1) in kb + 2 (mod 3)
     for (int j = 0; j < n_tiles; ++j) {
-        const int kb1 = kb == 2 ? 0 : kb + 1;
-        const int kb2 = kb1 == 2 ? 0 : kb1 + 1;
-        stage_k(j + 2, kb2);           // K'(j+2) replaces K'(j-1), V(j+1) replaces V(j-2): both idle since the
-        stage_v(j + 1, kb1);           // last barrier; the data is first read after the next one
+        const int kb = j & 3, kb1 = (j + 1) & 3, kb2 = (j + 2) & 3, kb3 = (j + 3) & 3;   // stage of tile j, j+1, ..
+#ifndef COME_EXP_NO_STAGE
+        load_bias(j + 3, kb3);
+        stage_k(j + 3, kb3);           // K'(j+3) replaces K'(j-1), V(j+2) replaces V(j-2): both idle since the
+        stage_v(j + 2, kb2);           // last barrier; they are first read two barriers from now
+#endif
 
-        const float sum0 = slot(0, 1, kb, kb2);        // slot a
+        const float sum0 = slot(0, 1, kb, kb3);        // slot a: V(j-1) lives in stage (j-1) & 3
         finish_slot(0, kb, sum0, j == 0);
         const float sum1 = slot(1, 0, kb1, kb);        // slot b
         finish_slot(1, kb, sum1, j == 0);
 
-        commit_bias(kb2);
-        staged_barrier();
-        kb = kb1;
+        // loads issued one iteration ago have landed; their raw bias becomes the K' block of tile j+2
+        staged_wait();
+#ifndef COME_EXP_NO_STAGE
+        commit_bias(j + 2, kb2);
+#endif
+#ifndef COME_EXP_NO_BARRIER
+        __syncthreads();
+#endif
     }
-    pv_mfma(1, kb == 0 ? 2 : kb - 1);      // V(n-1)
+    pv_mfma(1, (n_tiles - 1) & 3);      // V(n-1)
 
     // ---- epilogue: normalise, write O (and LSE)
 #pragma unroll
