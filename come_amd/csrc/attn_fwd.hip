@@ -329,8 +329,8 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnArgs a) {
 // Q is multiplied by c once (and rounded back to 16 bit); bias log2(e) and the reference point m of
 // the row ride through the fifth k-step as exact three-term 16-bit splits (K' carries the bias terms
 // and ones, Q' carries ones and the terms of -m).  m is the row maximum of the first key tile and is
-// moved only when a tile's row sum leaves a safe range (probabilities are then rescaled exactly as
-// in the usual online softmax); softmax is invariant to the choice of m, and fp32 / 16-bit floats
+// moved, by a power of two, only when a half-tile's row sum leaves a safe range (sums and outputs are
+// then rescaled as in the usual online softmax); softmax is invariant to the choice of m, and fp32 / 16-bit floats
 // keep full relative precision for probabilities above 1.  The steady state therefore spends one
 // exp2, half a pack and half a dot per score on the vector ALU and nothing else.
 // -------------------------------------------------------------------------------------
@@ -432,7 +432,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
     const uint32_t k_last = static_cast<uint32_t>(L - 1) * k_rs_b, v_last = static_cast<uint32_t>(L - 1) * v_rs_b;
     const uint32_t k_tile_step = static_cast<uint32_t>(kBlockN) * k_rs_b, v_tile_step = static_cast<uint32_t>(kBlockN) * v_rs_b;
 
-    auto stage_k = [&](int tile, int buf) {
+    auto stage_k = [&](int tile, int buf) __attribute__((always_inline)) {
         const int n0 = tile * kBlockN;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -442,13 +442,13 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
     };
     // raw bias of the 64 keys of a tile: wavefront 0 brings the aligned 32-bit word that holds each key's
     // 16-bit bias; it is converted into the fifth k-step block one iteration later (commit_bias)
-    auto load_bias = [&](int tile, int buf) {
+    auto load_bias = [&](int tile, int buf) __attribute__((always_inline)) {
         if (wave_u == 0 && b_seg) {
             const uint32_t key = static_cast<uint32_t>(min(tile * kBlockN + lane, L - 1));
             dma_b32(b_seg, ((b_mis + 2u * key) & ~3u), lds_address(&lds_braw[buf][0]));
         }
     };
-    auto stage_v = [&](int tile, int buf) {
+    auto stage_v = [&](int tile, int buf) __attribute__((always_inline)) {
         const int n0 = tile * kBlockN;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -457,7 +457,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
         }
     };
     // exact three-term 16-bit split of an fp32 value (an infinite value stays one term)
-    auto split3 = [&](float t, uint32_t &t_hi, uint32_t &t_mid, uint32_t &t_lo) {
+    auto split3 = [&](float t, uint32_t &t_hi, uint32_t &t_mid, uint32_t &t_lo) __attribute__((always_inline)) {
         t_hi = E::from_f32(t);
         t_mid = 0;
         t_lo = 0;
@@ -468,7 +468,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
             t_lo = E::from_f32(r1 - E::to_f32(static_cast<uint16_t>(t_mid)));
         }
     };
-    auto commit_bias = [&](int tile, int buf) {
+    auto commit_bias = [&](int tile, int buf) __attribute__((always_inline)) {
         if (wave_u == 0) {
             // [bias log2(e) in three terms | 1 1 1 | 0 0] then 16 bytes of zeros; -inf beyond the segment
             const int key = tile * kBlockN + lane;
@@ -492,14 +492,14 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
     };
     // the loads issued one iteration ago have landed (only the four direct loads of this iteration, plus
     // the bias load in wavefront 0, may still be in flight), then the workgroup meets
-    auto staged_wait = [&]() {
+    auto staged_wait = [&]() __attribute__((always_inline)) {
         if (wave_u == 0 && b_seg) {
             asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
         } else {
             asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
         }
     };
-    auto staged_barrier = [&](bool) {
+    auto staged_barrier = [&](bool) __attribute__((always_inline)) {
         staged_wait();
         __syncthreads();
     };
@@ -517,9 +517,12 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
                    (((4 * dt + 2 * ((lane >> 4) & 1) + ((i16 & 3) >> 1)) ^ (((i16 >> 3) & 1) << 2)) << 3) + 4 * (i16 & 1);
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-    f32x16 s_acc[2][2];          // S'' of the two query tiles (two 32-key halves each)
-    f32x16 o_acc[2][2];
-    u32x4 p_frag[2][4];
+    // s_acc[b][qt]: S'' of query tile qt for one 32-key half-tile; buffer b alternates between "being
+    // turned into probabilities" and "being built by the matrix pipe".  p_frag[b][qt][u]: the
+    // probabilities of that half-tile as B operands (u = 16-key step).
+    f32x16 s_acc[2][2];
+    f32x16 o_acc[2][2];          // [query tile][head-dim half]
+    u32x4 p_frag[2][2][2];
     float m_run[2] = {0.f, 0.f};  // reference point of the row, log2 units
     float l_run[2] = {0.f, 0.f};  // per-lane partial row sum
 #pragma unroll
@@ -527,150 +530,194 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
         o_acc[qt][0] = zero16;
         o_acc[qt][1] = zero16;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) p_frag[qt][u] = zero4();
+        for (int b = 0; b < 2; ++b) {
+            p_frag[b][qt][0] = zero4();
+            p_frag[b][qt][1] = zero4();
+        }
     }
 
-    auto score_mfma = [&](int qt, int buf) {
+    // scores of both query tiles against half-tile `half` of the K' tile in `buf`, into buffer b
+    auto score_mfma = [&](int b, int buf, int half) __attribute__((always_inline)) {
 #pragma unroll
         for (int ks = 0; ks < 5; ++ks) {
-            const uint16_t *kp = ks < 4 ? &lds_k[buf][k_rd[ks < 4 ? ks : 0]] : &lds_b[buf][b_rd];
-            const u32x4 kf0 = *reinterpret_cast<const u32x4 *>(kp);
-            const u32x4 kf1 = *reinterpret_cast<const u32x4 *>(kp + 32 * (ks < 4 ? kHeadDim : kBiasPitch));
-            const u32x4 qb = ks < 4 ? qf[qt][ks < 4 ? ks : 0] : q_ext[qt];
-            s_acc[qt][0] = E::mfma(kf0, qb, ks == 0 ? zero16 : s_acc[qt][0]);
-            s_acc[qt][1] = E::mfma(kf1, qb, ks == 0 ? zero16 : s_acc[qt][1]);
+            const uint16_t *kp = ks < 4 ? &lds_k[buf][k_rd[ks < 4 ? ks : 0] + 32 * half * kHeadDim]
+                                        : &lds_b[buf][b_rd + 32 * half * kBiasPitch];
+            const u32x4 kf = *reinterpret_cast<const u32x4 *>(kp);
+#pragma unroll
+            for (int qt = 0; qt < 2; ++qt)
+                s_acc[b][qt] = E::mfma(kf, ks < 4 ? qf[qt][ks < 4 ? ks : 0] : q_ext[qt], ks == 0 ? zero16 : s_acc[b][qt]);
         }
     };
-    auto pv_mfma = [&](int qt, int buf) {
+    // O^T += V^T P^T of both query tiles for half-tile `half` of the V tile in `buf`, probabilities of buffer b
+    auto pv_mfma = [&](int b, int buf, int half) __attribute__((always_inline)) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < 2; ++u) {
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt) {
-                const uint16_t *vp = &lds_v[buf][v_rd[dt] + (16 * u) * kHeadDim];
+                const uint16_t *vp = &lds_v[buf][v_rd[dt] + (32 * half + 16 * u) * kHeadDim];
                 const u32x2 lo2 = __builtin_bit_cast(u32x2, lds_read_tr(vp));
                 const u32x2 hi2 = __builtin_bit_cast(u32x2, lds_read_tr(vp + 8 * kHeadDim));
-                o_acc[qt][dt] = E::mfma(u32x4{lo2[0], lo2[1], hi2[0], hi2[1]}, p_frag[qt][u], o_acc[qt][dt]);
+                const u32x4 vf = u32x4{lo2[0], lo2[1], hi2[0], hi2[1]};
+#pragma unroll
+                for (int qt = 0; qt < 2; ++qt) o_acc[qt][dt] = E::mfma(vf, p_frag[b][qt][u], o_acc[qt][dt]);
             }
         }
     };
 
-    // One slot in explicit issue order.  The matrix pipe works on query tile Y: 10 score MFMAs against
-    // the K' tile in `kbuf` (S[Y] is rebuilt), then 8 P V MFMAs with the V tile in `vbuf` (P[Y] from the
-    // previous slot).  The vector ALU turns S[X] into P[X] in between: every MFMA is followed by a
-    // chunk of vector work, and the LDS reads of MFMA i + 2 are requested before it, so an in-order
-    // wavefront always has independent vector work behind each MFMA.  sched_barrier keeps the compiler
-    // from regrouping the chunks.  Returns the tile row sum of this lane.
-    auto slot = [&](int X, int Y, int kbuf, int vbuf) -> float {
-        u32x4 frag[18];
-        auto request = [&](int i) {
-            if (i < 10) {
-                const int ks = i >> 1, mt = i & 1;
-                frag[i] = ks < 4 ? *reinterpret_cast<const u32x4 *>(&lds_k[kbuf][k_rd[ks < 4 ? ks : 0] + 32 * mt * kHeadDim])
-                                 : *reinterpret_cast<const u32x4 *>(&lds_b[kbuf][b_rd + 32 * mt * kBiasPitch]);
-            } else if (i < 18) {
-                const int u = (i - 10) >> 1, dt = (i - 10) & 1;
-                const uint16_t *vp = &lds_v[vbuf][v_rd[dt] + (16 * u) * kHeadDim];
+    // One slot in explicit issue order.  The vector ALU turns the scores in buffer X (one 32-key half-tile,
+    // both query tiles) into probabilities.  Meanwhile the matrix pipe builds the scores of the next
+    // half-tile in buffer Y (10 MFMAs on 5 K' fragments, each fragment shared by both query tiles) and
+    // adds the previous half-tile's P V (8 MFMAs on 4 V fragments, probabilities of buffer Y from the
+    // previous slot).  Every MFMA is followed by a chunk of vector work and fragments are requested two
+    // fragments (four MFMAs) ahead, so an in-order wavefront always has independent work behind each
+    // MFMA.  sched_barrier keeps the compiler from regrouping the chunks.
+    // Returns through sum[qt] the row sums of this lane over the half-tile.
+    auto slot = [&](int X, int Y, int kbuf, int khalf, int vbuf, int vhalf, float (&sum)[2]) __attribute__((always_inline)) {
+        // fragments 0..3: V (u, dt) of the P V MFMAs 0..7; fragments 4..8: K' k-steps of the score MFMAs 8..17.
+        // P V goes first: the probabilities of buffer Y die while those of buffer X are born, and the score
+        // registers of buffer Y are not needed before half of buffer X has been consumed.
+        u32x4 frag[9];
+        auto request = [&](int f) __attribute__((always_inline)) {
+            if (f < 4) {
+                const int u = f >> 1, dt = f & 1;
+                const uint16_t *vp = &lds_v[vbuf][v_rd[dt] + (32 * vhalf + 16 * u) * kHeadDim];
                 const u32x2 lo2 = __builtin_bit_cast(u32x2, lds_read_tr(vp));
                 const u32x2 hi2 = __builtin_bit_cast(u32x2, lds_read_tr(vp + 8 * kHeadDim));
-                frag[i] = u32x4{lo2[0], lo2[1], hi2[0], hi2[1]};
+                frag[f] = u32x4{lo2[0], lo2[1], hi2[0], hi2[1]};
+            } else if (f < 9) {
+                const int ks = f - 4;
+                frag[f] = ks < 4 ? *reinterpret_cast<const u32x4 *>(&lds_k[kbuf][k_rd[ks < 4 ? ks : 0] + 32 * khalf * kHeadDim])
+                                 : *reinterpret_cast<const u32x4 *>(&lds_b[kbuf][b_rd + 32 * khalf * kBiasPitch]);
             }
         };
-        auto issue = [&](int i) {
-            if (i < 10) {
-                const int ks = i >> 1, mt = i & 1;
-                const u32x4 qb = ks < 4 ? qf[Y][ks < 4 ? ks : 0] : q_ext[Y];
-                s_acc[Y][mt] = E::mfma(frag[i], qb, ks == 0 ? zero16 : s_acc[Y][mt]);
+        auto issue = [&](int m) __attribute__((always_inline)) {
+            const int f = m >> 1, qt = m & 1;
+            // empty asm statements are ordering pins: MFMAs and exponentials are pure operations which the
+            // compiler would otherwise float out of their chunk (sched_barrier only fences what is already there)
+#ifndef COME_EXP_NO_FRAG_PIN
+            if (qt == 0) asm volatile("" : "+v"(frag[f]));
+#endif
+            if (f < 4) {
+                const int u = f >> 1, dt = f & 1;
+                o_acc[qt][dt] = E::mfma(frag[f], p_frag[Y][qt][u], o_acc[qt][dt]);
             } else {
-                const int u = (i - 10) >> 1, dt = (i - 10) & 1;
-                o_acc[Y][dt] = E::mfma(frag[i], p_frag[Y][u], o_acc[Y][dt]);
+                const int ks = f - 4;
+                s_acc[Y][qt] = E::mfma(frag[f], ks < 4 ? qf[qt][ks < 4 ? ks : 0] : q_ext[qt], ks == 0 ? zero16 : s_acc[Y][qt]);
             }
         };
         request(0);
         request(1);
-        float sum = 0.f;
+        sum[0] = 0.f;
+        sum[1] = 0.f;
         float p0 = 0.f, p1 = 0.f;
 #pragma unroll
         for (int c = 0; c < 16; ++c) {
-            issue(c);
-            request(c + 2);
-            if (c > 0) {                    // pack and add the pair whose exponentials were issued one chunk ago
-                const int pc = c - 1;
-                const uint32_t pw = E::pack2(p0, p1);
-                p_frag[X][pc >> 2][pc & 3] = pw;
-                sum = E::dot2_ones(pw, sum);
+            // MFMAs 0,1 | 2,3 | 4 | 5 | ... | 17: the last score MFMA is one chunk away from the end of the slot
+            if (c == 0) {
+                issue(0);
+                issue(1);
+                request(2);
+            } else if (c == 1) {
+                issue(2);
+                issue(3);
+                request(3);
+            } else {
+                issue(c + 2);
+                if ((c & 1) == 0) request((c >> 1) + 3);     // chunk 2 -> fragment 4, ..., chunk 10 -> fragment 8
             }
-            p0 = __builtin_amdgcn_exp2f(s_acc[X][c >> 3][2 * (c & 7)]);
-            p1 = __builtin_amdgcn_exp2f(s_acc[X][c >> 3][2 * (c & 7) + 1]);
+            if (c > 0) {                    // pack and add the pair whose exponentials were issued one chunk ago
+                const int pc = c - 1, qt = pc >> 3, w = pc & 7;
+                const uint32_t pw = E::pack2(p0, p1);
+                p_frag[X][qt][w >> 2][w & 3] = pw;
+                sum[qt] = E::dot2_ones(pw, sum[qt]);
+            }
+            float s0 = s_acc[X][c >> 3][2 * (c & 7)], s1 = s_acc[X][c >> 3][2 * (c & 7) + 1];
+#ifndef COME_EXP_NO_S_PIN
+            asm volatile("" : "+v"(s0), "+v"(s1));
+#endif
+            p0 = __builtin_amdgcn_exp2f(s0);
+            p1 = __builtin_amdgcn_exp2f(s1);
+#ifndef COME_EXP_NO_P_PIN
+            asm volatile("" : "+v"(p0), "+v"(p1));
+#endif
             __builtin_amdgcn_sched_barrier(0);
         }
-        issue(16);
         {
             const uint32_t pw = E::pack2(p0, p1);
-            p_frag[X][3][3] = pw;
-            sum = E::dot2_ones(pw, sum);
+            p_frag[X][1][1][3] = pw;
+            sum[1] = E::dot2_ones(pw, sum[1]);
         }
-        issue(17);
         // the decision that follows the slot is tied to its end, so that the branch cannot be moved
         // above the probability chunks
-        float sum_late = sum;
-        asm volatile("" : "+v"(sum_late) : "v"(p_frag[X][3][3]));
-        return sum_late;
+        asm volatile("" : "+v"(sum[1]) : "v"(p_frag[X][1][1][3]));
     };
 
-    // Exact path of query tile X: move the reference point to the row maximum of this tile and redo its
-    // probabilities.  The scores are rebuilt from the K' tile (still in LDS) rather than kept alive
-    // through the slot, which would cost 32 registers in the steady state for a path that is almost
-    // never taken.
-    auto recentre = [&](int X, int kbuf) {
-        score_mfma(X, kbuf);
-        float mx = s_acc[X][0][0];
-#pragma unroll
-        for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s_acc[X][0][e]);
-#pragma unroll
-        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[X][1][e]);
-        mx = max_across_halves(mx);
-        const float delta = mx == -INFINITY ? 0.f : mx;          // every key masked so far: stay put
-        float sum = 0.f;
-#pragma unroll
-        for (int c = 0; c < 16; ++c) {
-            const float p0 = __builtin_amdgcn_exp2f(s_acc[X][c >> 3][2 * (c & 7)] - delta);
-            const float p1 = __builtin_amdgcn_exp2f(s_acc[X][c >> 3][2 * (c & 7) + 1] - delta);
-            const uint32_t pw = E::pack2(p0, p1);
-            p_frag[X][c >> 2][c & 3] = pw;
-            sum = E::dot2_ones(pw, sum);
-            __builtin_amdgcn_sched_barrier(0);      // rare path: keep it serial and small in registers
+    // writes the three-term split of -m_run[qt] into the fifth k-step of Q'
+    auto publish_reference = [&](int qt) __attribute__((always_inline)) {
+        uint32_t n_hi, n_mid, n_lo;
+        split3(-m_run[qt], n_hi, n_mid, n_lo);
+        if (h == 0) {
+            q_ext[qt][1] = E::kOne | (n_hi << 16);
+            q_ext[qt][2] = n_mid | (n_lo << 16);
         }
-        const float alpha = __builtin_amdgcn_exp2f(fminf(-delta, 126.f));   // what was accumulated so far shrinks
-        // in-place multiplies: written as asm so that the accumulator tuples keep their registers across
-        // this rarely taken branch (a plain multiply makes the allocator copy both 16-register tuples)
+    };
+    // O[qt] *= f, in place.  Written as asm so that the accumulator tuples keep their registers across a
+    // rarely taken branch (plain arithmetic makes the register allocator copy the 16-register tuples).
+    auto scale_o = [&](int qt, float f) __attribute__((always_inline)) {
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                float t = o_acc[X][dt][e];
-                asm volatile("v_mul_f32 %0, %1, %0" : "+v"(t) : "v"(alpha));
-                o_acc[X][dt][e] = t;
+                float t = o_acc[qt][dt][e];
+                asm volatile("v_mul_f32 %0, %1, %0" : "+v"(t) : "v"(f));
+                o_acc[qt][dt][e] = t;
             }
-        l_run[X] = l_run[X] * alpha + sum;
-        m_run[X] += delta;
-        uint32_t n_hi, n_mid, n_lo;
-        split3(-m_run[X], n_hi, n_mid, n_lo);
-        if (h == 0) {
-            q_ext[X][1] = E::kOne | (n_hi << 16);
-            q_ext[X][2] = n_mid | (n_lo << 16);
-        }
     };
-    auto finish_slot = [&](int X, int kbuf, float sum, bool force) {
-        if (force || __any(!(sum <= kSumLimit))) {
-            recentre(X, kbuf);
+
+    // End of a slot.  Steady state: add the half-tile row sums.  Rare path, taken when a row sum left the
+    // safe range: the reference point of such rows moves up by a power of two, 2^shift.
+    //  - the scores of the next half-tile (buffer Y, built against the old reference) are shifted now;
+    //  - the row sum is rescaled now;
+    //  - O is rescaled one slot later (o_pending), after the P V MFMAs of the probabilities just made,
+    //    which are relative to the old reference, have been accumulated.
+    float o_pending[2] = {1.f, 1.f};
+    bool any_pending = false;                  // wave-uniform
+    auto finish_slot = [&](int Y, const float (&sum)[2]) __attribute__((always_inline)) {
+        const bool bad = !(sum[0] <= kSumLimit) || !(sum[1] <= kSumLimit);
+        if (__any(bad) || any_pending) {
+            // the asm arithmetic below reads MFMA results; the compiler cannot see that, so the wait states an
+            // MFMA result needs before a vector instruction may read it are spent here explicitly
+            asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+            bool again = false;
+#pragma unroll
+            for (int qt = 0; qt < 2; ++qt) {
+                scale_o(qt, o_pending[qt]);
+                int shift = sum[qt] <= kSumLimit ? 0 : max(__builtin_amdgcn_frexp_expf(sum[qt]) - 2, 1);
+                shift = static_cast<int>(max_across_halves(static_cast<float>(shift)));   // both half-waves of a row agree
+                const float down = __builtin_amdgcn_exp2f(static_cast<float>(-shift));
+                const float fshift = static_cast<float>(shift);
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    float t = s_acc[Y][qt][e];
+                    asm volatile("v_sub_f32 %0, %0, %1" : "+v"(t) : "v"(fshift));
+                    s_acc[Y][qt][e] = t;
+                }
+                l_run[qt] = (l_run[qt] + sum[qt]) * down;
+                m_run[qt] += fshift;
+                publish_reference(qt);
+                o_pending[qt] = down;
+                again = again || __any(shift != 0);
+            }
+            any_pending = again;
         } else {
-            l_run[X] += sum;
+            l_run[0] += sum[0];
+            l_run[1] += sum[1];
         }
     };
 
     // ---- prologue
     const int n_tiles = (L + kBlockN - 1) / kBlockN;
-    {   // the last V stage stands in for "tile -1": zeros (P1 is zero there as well)
+    {   // the last V stage stands in for "tile -1": zeros (its probabilities are zero as well)
         u32x4 *z = reinterpret_cast<u32x4 *>(&lds_v[kStages - 1][0]);
         for (int i = tid; i < kBlockN * kHeadDim / 8; i += kThreads) z[i] = zero4();
     }
@@ -686,7 +733,18 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
     stage_k(2, 2);
     stage_v(1, 1);
     staged_barrier(false);             // everything but this last group has landed
-    score_mfma(0, 0);
+    // reference point of every row: its maximum over the first 32 keys (0 if all of them are masked)
+    score_mfma(0, 0, 0);
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+        float mx = s_acc[0][qt][0];
+#pragma unroll
+        for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s_acc[0][qt][e]);
+        mx = max_across_halves(mx);
+        m_run[qt] = (mx == -INFINITY || mx != mx) ? 0.f : mx;
+        publish_reference(qt);
+    }
+    score_mfma(0, 0, 0);               // the same scores, now relative to the reference
 
     for (int j = 0; j < n_tiles; ++j) {
         const int kb = j & 3, kb1 = (j + 1) & 3, kb2 = (j + 2) & 3, kb3 = (j + 3) & 3;   // stage of tile j, j+1, ..
@@ -695,11 +753,13 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
         stage_k(j + 3, kb3);           // K'(j+3) replaces K'(j-1), V(j+2) replaces V(j-2): both idle since the
         stage_v(j + 2, kb2);           // last barrier; they are first read two barriers from now
 #endif
-
-        const float sum0 = slot(0, 1, kb, kb3);        // slot a: V(j-1) lives in stage (j-1) & 3
-        finish_slot(0, kb, sum0, j == 0);
-        const float sum1 = slot(1, 0, kb1, kb);        // slot b
-        finish_slot(1, kb, sum1, j == 0);
+        float sum[2];
+        // slot a: keys 0..31 of tile j become probabilities; scores of keys 32..63; P V of keys 32..63 of tile j-1
+        slot(0, 1, kb, 1, kb3, 1, sum);
+        finish_slot(1, sum);
+        // slot b: keys 32..63 of tile j become probabilities; scores of keys 0..31 of tile j+1; P V of keys 0..31 of tile j
+        slot(1, 0, kb1, 0, kb, 0, sum);
+        finish_slot(0, sum);
 
         // loads issued one iteration ago have landed; their raw bias becomes the K' block of tile j+2
         staged_wait();
@@ -710,7 +770,13 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
         __syncthreads();
 #endif
     }
-    pv_mfma(1, (n_tiles - 1) & 3);      // V(n-1)
+    pv_mfma(1, (n_tiles - 1) & 3, 1);      // keys 32..63 of the last tile
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o_acc[qt][dt][e] *= o_pending[qt];
 
     // ---- epilogue: normalise, write O (and LSE)
 #pragma unroll

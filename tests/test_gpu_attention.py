@@ -122,6 +122,41 @@ def test_count_bias_equals_key_duplication():
     assert float(diff.max()) <= 2e-2 and float(diff.mean()) <= 2e-3
 
 
+@pytest.mark.parametrize("kind", ["ramp", "jump", "late_rows", "descending"])
+def test_reference_point_moves(kind):
+    """Scores that grow by many orders of magnitude along the keys: the kernel keeps probabilities relative
+    to a per-row reference point taken from the first keys and has to move it (rare path) without losing
+    accuracy.  Checked against the closed form like every other case."""
+    L, H = 1500, 2
+    qkv = torch.randn(L, 3, H, 64).bfloat16()
+    if kind == "ramp":
+        bias = torch.linspace(-30.0, 30.0, L)
+    elif kind == "jump":
+        bias = torch.zeros(L)
+        bias[700], bias[701], bias[1333] = 40.0, 25.0, 55.0
+    elif kind == "late_rows":
+        bias = torch.zeros(L)
+        qkv[:, 1, :, :] *= torch.linspace(0.2, 6.0, L)[:, None, None].bfloat16()     # later keys score far higher
+    else:
+        bias = torch.linspace(40.0, -40.0, L)
+    bias = bias.bfloat16()
+    cu = _cu([L])
+    ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias)
+    out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), L, perkey_bias=bias.to(DEV),
+                                                                 return_attn_probs=True)
+    assert bool(torch.isfinite(out).all())
+    if kind == "late_rows":
+        # logits of up to +-35 nats with near-ties between the leading keys: the kernel multiplies Q by
+        # softmax_scale * log2(e) once and rounds it back to 16 bit, an error in the logit that grows with its
+        # magnitude (about 1e-3 * |logit| / sqrt(head_dim) bits); at this extreme it shows as a few 1e-2
+        diff = (out.float().cpu() - ref).abs()
+        assert float(diff.max()) <= 8e-2 and float(diff.mean()) <= 5e-3, (float(diff.max()), float(diff.mean()))
+        torch.testing.assert_close(lse.cpu(), ref_lse, atol=5e-2, rtol=2e-3)
+        return
+    _compare(out, ref)
+    torch.testing.assert_close(lse.cpu(), ref_lse, atol=5e-3, rtol=1e-3)
+
+
 def test_strided_views_and_separate_tensors():
     lens, H = [90, 41], 4
     P = sum(lens)
