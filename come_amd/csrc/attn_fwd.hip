@@ -434,14 +434,17 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
 
     auto stage_k = [&](int tile, int buf) __attribute__((always_inline)) {
         const int n0 = tile * kBlockN;
+        const uint32_t tile_off = static_cast<uint32_t>(tile) * k_tile_step;         // wave-uniform
+        const bool full = n0 + kBlockN <= L;                                        // wave-uniform
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const uint32_t off = n0 + st_row[i] < L ? static_cast<uint32_t>(tile) * k_tile_step + k_goff[i] : k_last + k_chunk[i];
+            uint32_t off = tile_off + k_goff[i];
+            if (!full) off = n0 + st_row[i] < L ? off : k_last + k_chunk[i];
             dma_b128(k_seg, off, lds_address(&lds_k[buf][(2 * wave_u + i) * 512]));
         }
     };
     // raw bias of the 64 keys of a tile: wavefront 0 brings the aligned 32-bit word that holds each key's
-    // 16-bit bias; it is converted into the fifth k-step block one iteration later (commit_bias)
+    // 16-bit bias; it is converted into the fifth k-step block two iterations later (commit_bias)
     auto load_bias = [&](int tile, int buf) __attribute__((always_inline)) {
         if (wave_u == 0 && b_seg) {
             const uint32_t key = static_cast<uint32_t>(min(tile * kBlockN + lane, L - 1));
@@ -450,9 +453,12 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
     };
     auto stage_v = [&](int tile, int buf) __attribute__((always_inline)) {
         const int n0 = tile * kBlockN;
+        const uint32_t tile_off = static_cast<uint32_t>(tile) * v_tile_step;
+        const bool full = n0 + kBlockN <= L;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const uint32_t off = n0 + st_row[i] < L ? static_cast<uint32_t>(tile) * v_tile_step + v_goff[i] : v_last + v_chunk[i];
+            uint32_t off = tile_off + v_goff[i];
+            if (!full) off = n0 + st_row[i] < L ? off : v_last + v_chunk[i];
             dma_b128(v_seg, off, lds_address(&lds_v[buf][(2 * wave_u + i) * 512]));
         }
     };
@@ -468,15 +474,20 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
             t_lo = E::from_f32(r1 - E::to_f32(static_cast<uint16_t>(t_mid)));
         }
     };
+    // conversion of the raw bias of one tile, split in two so that the LDS read is in flight during a slot:
+    // peek_bias() requests the word, commit_bias() converts it and writes the fifth k-step block
+    // [bias log2(e) in three terms | 1 1 1 | 0 0] followed by 16 bytes of zeros; -inf beyond the segment
+    uint32_t b_word = 0;
+    auto peek_bias = [&](int buf) __attribute__((always_inline)) {
+        if (wave_u == 0 && b_seg) b_word = lds_braw[buf][lane];
+    };
     auto commit_bias = [&](int tile, int buf) __attribute__((always_inline)) {
         if (wave_u == 0) {
-            // [bias log2(e) in three terms | 1 1 1 | 0 0] then 16 bytes of zeros; -inf beyond the segment
             const int key = tile * kBlockN + lane;
             float bias = 0.f;
             if (b_seg) {
-                const uint32_t word = lds_braw[buf][lane];
                 const uint32_t at = b_mis + 2u * static_cast<uint32_t>(min(key, L - 1));
-                bias = E::to_f32(static_cast<uint16_t>((at & 2u) ? (word >> 16) : (word & 0xffffu)));
+                bias = E::to_f32(static_cast<uint16_t>((at & 2u) ? (b_word >> 16) : (b_word & 0xffffu)));
             }
             uint32_t t_hi, t_mid, t_lo;
             split3(bias * kLog2e, t_hi, t_mid, t_lo);
@@ -490,18 +501,12 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
             *reinterpret_cast<u32x4 *>(&lds_b[buf][lane * kBiasPitch + 8]) = zero4();
         }
     };
-    // the loads issued one iteration ago have landed (only the four direct loads of this iteration, plus
-    // the bias load in wavefront 0, may still be in flight), then the workgroup meets
-    auto staged_wait = [&]() __attribute__((always_inline)) {
-        if (wave_u == 0 && b_seg) {
+    auto staged_wait = [&](bool with_bias_load) __attribute__((always_inline)) {
+        if (with_bias_load && wave_u == 0 && b_seg) {
             asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
         } else {
             asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
         }
-    };
-    auto staged_barrier = [&](bool) __attribute__((always_inline)) {
-        staged_wait();
-        __syncthreads();
     };
 
     // LDS read offsets (in elements) of this lane
@@ -592,6 +597,9 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
         };
         auto issue = [&](int m) __attribute__((always_inline)) {
             const int f = m >> 1, qt = m & 1;
+#ifdef COME_EXP_NO_MFMA
+            if (f >= 0) return;
+#endif
             // empty asm statements are ordering pins: MFMAs and exponentials are pure operations which the
             // compiler would otherwise float out of their chunk (sched_barrier only fences what is already there)
 #ifndef COME_EXP_NO_FRAG_PIN
@@ -632,11 +640,16 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
                 sum[qt] = E::dot2_ones(pw, sum[qt]);
             }
             float s0 = s_acc[X][c >> 3][2 * (c & 7)], s1 = s_acc[X][c >> 3][2 * (c & 7) + 1];
-#ifndef COME_EXP_NO_S_PIN
+#ifdef COME_EXP_S_PIN
             asm volatile("" : "+v"(s0), "+v"(s1));
 #endif
+#ifdef COME_EXP_NO_EXP
+            p0 = s0;
+            p1 = s1;
+#else
             p0 = __builtin_amdgcn_exp2f(s0);
             p1 = __builtin_amdgcn_exp2f(s1);
+#endif
 #ifndef COME_EXP_NO_P_PIN
             asm volatile("" : "+v"(p0), "+v"(p1));
 #endif
@@ -692,7 +705,9 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
 #pragma unroll
             for (int qt = 0; qt < 2; ++qt) {
                 scale_o(qt, o_pending[qt]);
-                int shift = sum[qt] <= kSumLimit ? 0 : max(__builtin_amdgcn_frexp_expf(sum[qt]) - 2, 1);
+                float row_sum = sum[qt];
+                asm volatile("" : "+v"(row_sum));       // keeps the arithmetic of this rare path inside the branch
+                int shift = row_sum <= kSumLimit ? 0 : max(__builtin_amdgcn_frexp_expf(row_sum) - 2, 1);
                 shift = static_cast<int>(max_across_halves(static_cast<float>(shift)));   // both half-waves of a row agree
                 const float down = __builtin_amdgcn_exp2f(static_cast<float>(-shift));
                 const float fshift = static_cast<float>(shift);
@@ -702,7 +717,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
                     asm volatile("v_sub_f32 %0, %0, %1" : "+v"(t) : "v"(fshift));
                     s_acc[Y][qt][e] = t;
                 }
-                l_run[qt] = (l_run[qt] + sum[qt]) * down;
+                l_run[qt] = (l_run[qt] + row_sum) * down;
                 m_run[qt] += fshift;
                 publish_reference(qt);
                 o_pending[qt] = down;
@@ -723,16 +738,20 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
     }
     load_bias(0, 0);
     load_bias(1, 1);
+    load_bias(2, 2);
+    load_bias(3, 3);
     stage_k(0, 0);
     stage_v(0, 0);
     stage_k(1, 1);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    peek_bias(0);
     commit_bias(0, 0);
+    peek_bias(1);
     commit_bias(1, 1);
-    load_bias(2, 2);                   // tiles of iteration 1 start their flight
-    stage_k(2, 2);
+    stage_k(2, 2);                     // tiles of iteration 1 start their flight
     stage_v(1, 1);
-    staged_barrier(false);             // everything but this last group has landed
+    staged_wait(false);                // everything but this last group has landed
+    __syncthreads();
     // reference point of every row: its maximum over the first 32 keys (0 if all of them are masked)
     score_mfma(0, 0, 0);
 #pragma unroll
@@ -749,25 +768,44 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
     for (int j = 0; j < n_tiles; ++j) {
         const int kb = j & 3, kb1 = (j + 1) & 3, kb2 = (j + 2) & 3, kb3 = (j + 3) & 3;   // stage of tile j, j+1, ..
 #ifndef COME_EXP_NO_STAGE
-        load_bias(j + 3, kb3);
+        load_bias(j + 4, kb);          // raw bias runs one more tile ahead (converted between the slots of iteration j+2)
         stage_k(j + 3, kb3);           // K'(j+3) replaces K'(j-1), V(j+2) replaces V(j-2): both idle since the
         stage_v(j + 2, kb2);           // last barrier; they are first read two barriers from now
 #endif
         float sum[2];
+        peek_bias(kb2);
+#ifdef COME_EXP_TIMING
+        const uint64_t t_a = __builtin_readcyclecounter();
+#endif
         // slot a: keys 0..31 of tile j become probabilities; scores of keys 32..63; P V of keys 32..63 of tile j-1
         slot(0, 1, kb, 1, kb3, 1, sum);
         finish_slot(1, sum);
+#ifndef COME_EXP_NO_STAGE
+        commit_bias(j + 2, kb2);       // raw bias landed before the last barrier; published by the next one
+#endif
         // slot b: keys 32..63 of tile j become probabilities; scores of keys 0..31 of tile j+1; P V of keys 0..31 of tile j
+#ifdef COME_EXP_TIMING
+        const uint64_t t_b = __builtin_readcyclecounter();
+#endif
         slot(1, 0, kb1, 0, kb, 0, sum);
         finish_slot(0, sum);
-
-        // loads issued one iteration ago have landed; their raw bias becomes the K' block of tile j+2
-        staged_wait();
-#ifndef COME_EXP_NO_STAGE
-        commit_bias(j + 2, kb2);
+#ifdef COME_EXP_TIMING
+        const uint64_t t_c = __builtin_readcyclecounter();
 #endif
+
+        staged_wait(true);             // loads issued one iteration ago have landed
 #ifndef COME_EXP_NO_BARRIER
         __syncthreads();
+#endif
+#ifdef COME_EXP_TIMING
+        if (a.lse && blockIdx.x == 1000 && lane == 0 && j >= 100 && j < 132) {
+            const uint64_t t_d = __builtin_readcyclecounter();
+            float *dump = a.lse + (wave * 32 + (j - 100)) * 4;
+            dump[0] = static_cast<float>(t_b - t_a);
+            dump[1] = static_cast<float>(t_c - t_b);
+            dump[2] = static_cast<float>(t_d - t_c);
+            dump[3] = static_cast<float>(t_d & 0xffffff);
+        }
 #endif
     }
     pv_mfma(1, (n_tiles - 1) & 3, 1);      // keys 32..63 of the last tile
