@@ -4,13 +4,27 @@
 // one window (or of one copied token), issues all of the window's loads back to back
 // (nine independent 16-byte loads for a 3x3 window) and writes either their mean
 // (merged) or the rows themselves (kept).  A wavefront therefore reads 1 KiB
-// contiguous per source row and writes 1 KiB contiguous per packed row.
+// contiguous per source row and writes 1 KiB contiguous per packed row.  Token data is
+// touched once, so loads and stores carry the non-temporal hint; the rows an unmerge
+// reads several times (merged windows) use ordinary loads and stay in L2.
 #include "come_common.h"
 
 namespace come {
 namespace {
 
 constexpr int kThreads = 256;
+
+// 16-byte global accesses; the streamed variants carry the non-temporal hint (data used once)
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ inline uint4 ld16(const uint4 *p) { return *p; }
+__device__ inline uint4 ld16_stream(const uint4 *p) {
+    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ inline void st16_stream(uint4 *p, const uint4 &v) {
+    const u32x4_t w = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(w, reinterpret_cast<u32x4_t *>(p));
+}
 
 struct MergeGeom {
     int rows, n_tok, start, groups;
@@ -136,7 +150,7 @@ __global__ __launch_bounds__(kThreads) void merge_vec_kernel(const MergeArgs a) 
             for (int dy = 0; dy < GH; ++dy)
 #pragma unroll
                 for (int dx = 0; dx < GW; ++dx)
-                    v[dy * GW + dx] = p[(static_cast<int64_t>(dy) * g.W + dx) * chunks];
+                    v[dy * GW + dx] = ld16_stream(p + (static_cast<int64_t>(dy) * g.W + dx) * chunks);
             if (merged) {
                 float acc[V::N];
 #pragma unroll
@@ -150,11 +164,11 @@ __global__ __launch_bounds__(kThreads) void merge_vec_kernel(const MergeArgs a) 
                 }
 #pragma unroll
                 for (int e = 0; e < V::N; ++e) acc[e] = acc[e] / static_cast<float>(GH * GW);
-                if (row0 < g.out_rows) dst[row0 * chunks + chunk] = V::pack(acc);
+                if (row0 < g.out_rows) st16_stream(dst + row0 * chunks + chunk, V::pack(acc));
             } else {
 #pragma unroll
                 for (int t = 0; t < GH * GW; ++t)
-                    if (row0 + t < g.out_rows) dst[(row0 + t) * chunks + chunk] = v[t];
+                    if (row0 + t < g.out_rows) st16_stream(dst + (row0 + t) * chunks + chunk, v[t]);
             }
         } else {
             if (merged) {
@@ -216,7 +230,7 @@ __global__ __launch_bounds__(kThreads) void merge_vec_kernel(const MergeArgs a) 
         row = static_cast<int64_t>(a.offsets[b + 1]) - g.tail + r;
     }
     const int64_t flat = static_cast<int64_t>(b) * g.n_tok + tok;
-    if (row < g.out_rows) dst[row * chunks + chunk] = src[flat * chunks + chunk];
+    if (row < g.out_rows) st16_stream(dst + row * chunks + chunk, ld16_stream(src + flat * chunks + chunk));
     if (chunk == 0) {
         note_row(a, flat, row);
         note_weight(a, row, 1);
@@ -319,7 +333,7 @@ __global__ __launch_bounds__(kThreads) void split_vec_kernel(const uint4 *__rest
     }
 #pragma unroll
     for (int r = 0; r < kSplitRows; ++r)
-        if (i0 + r < total) out[(i0 + r) * chunks + chunk] = v[r];
+        if (i0 + r < total) st16_stream(out + (i0 + r) * chunks + chunk, v[r]);
 }
 
 template <typename IndexT>
