@@ -12,8 +12,8 @@ C = 1024, bf16, 3x3 windows, ratio 0.5) as GB/s of algorithmic bytes with its ow
 the select + plan + merge pipeline rate.
 
 ``roofline`` times the dominant kernel with HIP events on the launch stream; ``cpu_baseline`` times
-the reference's PyTorch CPU path (SDPA with the bias as attn_mask) on a bounded sample of the same
-workload on the host cores.
+the reference's PyTorch CPU path (SDPA with the bias as attn_mask) on the same workload on the host
+cores, stopped after about 20 s of work.
 """
 
 from __future__ import annotations
@@ -32,6 +32,15 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0       # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 
+# HBM bytes per launch of each kernel on exactly the workloads built below, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE passes (KiB per dispatch), FETCH_SIZE scaled by 2.000 and WRITE_SIZE by 1.000 -- the factors a 256 MiB
+# device copy (``--only copy``) gives for the same counters.  The summaries are in profiles/.
+TRAFFIC_BYTES = {
+    "attn": int((392103 * 2.000 + 97738) * 1024),
+    "merge": int((22095 * 2.000 + 25836) * 1024),
+    "unmerge": int((16124 * 2.000 + 44046) * 1024),
+}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -40,7 +49,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "copy"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -207,13 +216,14 @@ def bench_merge_unmerge(device, iters=200, warmup=20):
                   "value": round(merge_gbs, 1), "unit": "GB/s", "us_per_call": round(merge_ms / iters * 1e3, 2),
                   "algorithmic_bytes": w["merge_bytes"], "iters": iters, "rotating_buffer_sets": 8,
                   "roofline": {"bound": "hbm", "achieved": round(merge_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                               "frac": round(merge_gbs / PEAK_HBM_GBS, 4), "traffic": None},
+                               "frac": round(merge_gbs / PEAK_HBM_GBS, 4), "traffic": TRAFFIC_BYTES["merge"]},
                   "select_plan_merge_us": round(pipe_ms / iters * 1e3, 2)},
         "unmerge": {"workload": "C2 unmerge: P=%d -> %d rows, C=1024 bf16" % (w["P"], w["frames"] * w["N"]),
                     "value": round(split_gbs, 1), "unit": "GB/s", "us_per_call": round(split_ms / iters * 1e3, 2),
                     "algorithmic_bytes": w["split_bytes"], "iters": iters, "rotating_buffer_sets": 8,
                     "roofline": {"bound": "hbm", "achieved": round(split_gbs, 1), "peak": PEAK_HBM_GBS,
-                                 "unit": "GB/s", "frac": round(split_gbs / PEAK_HBM_GBS, 4), "traffic": None}},
+                                 "unit": "GB/s", "frac": round(split_gbs / PEAK_HBM_GBS, 4),
+                                 "traffic": TRAFFIC_BYTES["unmerge"]}},
     }
 
 
@@ -221,34 +231,35 @@ def bench_merge_unmerge(device, iters=200, warmup=20):
 # host-CPU baseline (the reference's PyTorch path on the CPU), bounded sample
 # ------------------------------------------------------------------------------------------
 
-def cpu_baseline_attention(w, q_rows=2048):
-    """SDPA in bf16 with the bias as attn_mask, the first ``q_rows`` queries of segment 0 against all of
-    its 25 536 keys, all 16 heads.  Same flop formula as the GPU figure (4 * rows * L * d * H)."""
+def cpu_baseline_attention(w, min_s=10.0, budget_s=20.0, q_chunk=4096):
+    """The reference's PyTorch CPU path for this operator (per segment, SDPA in bf16 with the bias as
+    attn_mask, queries in chunks of ``q_chunk``) over the same workload, repeated until ``min_s`` seconds are
+    sampled and stopped after ``budget_s``.  Same flop formula as the GPU figure (4 * rows * L * d * H per chunk)."""
     import torch
     import oracle
 
-    cores = os.cpu_count() or 1
-    threads = min(cores, 16)
+    threads = min(os.cpu_count() or 1, 16)
     torch.set_num_threads(threads)
-    L = w["lens"][0]
-    qkv = w["qkv"][:L].cpu()
-    bias = w["bias"][:L].cpu()
-    # the oracle's SDPA leg works on whole segments; restrict the queries by packing a view
-    q, k, v = qkv.unbind(1)
-    mask = bias[None, None, None, :]
-    kh, vh = k.transpose(0, 1).unsqueeze(0), v.transpose(0, 1).unsqueeze(0)
-    qh = q[:q_rows].transpose(0, 1).unsqueeze(0)
-    times = []
-    for _ in range(3):
-        t0 = time.perf_counter()
-        torch.nn.functional.scaled_dot_product_attention(qh, kh, vh, attn_mask=mask, scale=0.125)
-        times.append(time.perf_counter() - t0)
-    t = sorted(times)[1]
-    flops = 4.0 * q_rows * L * w["D"] * w["H"]
-    del oracle
-    return {"value": round(flops / t / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"torch SDPA bf16 + attn_mask bias, first {q_rows} queries of segment 0 x all {L} keys x 16 heads,"
-                      f" median of 3 ({t:.2f} s each)"}
+    qkv, bias = w["qkv"].cpu(), w["bias"].cpu()
+    bounds = [0, w["lens"][0], w["lens"][0] + w["lens"][1]]
+    flops, spent, rows, passes = 0.0, 0.0, 0, 0
+    while spent < min_s:                                       # whole passes until enough time is sampled
+        for s, e in zip(bounds[:-1], bounds[1:]):
+            for c0 in range(s, e, q_chunk):
+                if spent >= budget_s:
+                    break
+                c1 = min(e, c0 + q_chunk)
+                t0 = time.perf_counter()
+                oracle.sdpa_bf16_chunk(qkv, bias, s, e, c0, c1, 0.125)
+                spent += time.perf_counter() - t0
+                flops += 4.0 * (c1 - c0) * (e - s) * w["D"] * w["H"]
+                rows += c1 - c0
+        passes += 1
+    total_rows = bounds[-1]
+    return {"value": round(flops / spent / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"torch CPU SDPA bf16 + attn_mask bias on the same workload, {rows} query rows of "
+                      f"{total_rows} per pass ({passes} passes; all keys of their segment, 16 heads) in {spent:.1f} s, "
+                      f"chunks of {q_chunk} queries"}
 
 
 def cpu_baseline_merge(mw):
@@ -296,7 +307,16 @@ def main():
     torch.cuda.set_device(device)
 
     if args.only:
-        if args.only == "attn":
+        if args.only == "copy":
+            # plain device copy of known size: the yardstick the HBM byte counters are scaled by
+            nbytes = 256 << 20
+            src = torch.empty(nbytes, dtype=torch.uint8, device=device).random_(0, 255)
+            dst = torch.empty_like(src)
+            _, ms = time_loop(lambda: dst.copy_(src), args.steps, args.warmup)
+            print(json.dumps({"only": "copy", "bytes_read": nbytes, "bytes_written": nbytes,
+                              "us_per_call": ms / args.steps * 1e3,
+                              "GBs": 2 * nbytes / (ms / args.steps * 1e-3) / 1e9}))
+        elif args.only == "attn":
             w, wall, ev_ms = bench_attention(args.steps, args.warmup, device)
             print(json.dumps({"only": "attn", "ms_per_call": ev_ms / args.steps,
                               "tflops": w["flops"] / (ev_ms / args.steps * 1e-3) / 1e12}))
@@ -334,8 +354,8 @@ def main():
                                "scale 0.125, non-causal",
                    "algorithmic_flops_per_step": w["flops"]},
         "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(kernel_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None,
-                     "kernel": "attn_fwd_kernel<bf16>", "ms_per_launch": round(ev_ms / args.steps, 4)},
+                     "frac": round(kernel_tflops / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES["attn"],
+                     "kernel": "attn_fwd_pipe_kernel<bf16>", "ms_per_launch": round(ev_ms / args.steps, 4)},
     }
     mw = None
     if not args.no_other:

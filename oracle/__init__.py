@@ -50,4 +50,5 @@ from .selection import (  # noqa: F401
 from .attention import (  # noqa: F401
     biased_varlen_attention,
     biased_varlen_attention_sdpa_bf16,
+    sdpa_bf16_chunk,
 )

@@ -79,3 +79,14 @@ def biased_varlen_attention_sdpa_bf16(
             o = torch.nn.functional.scaled_dot_product_attention(qh, kh, vh, attn_mask=mask, scale=scale)
             out[c0:c1] = o[0].transpose(0, 1)
     return out
+
+
+def sdpa_bf16_chunk(qkv, perkey_bias, seg_start: int, seg_end: int, q_start: int, q_end: int, scale: float):
+    """One query chunk ``[q_start, q_end)`` of the CPU baseline above against all keys of its segment
+    ``[seg_start, seg_end)``; lets a caller bound the time it spends."""
+    q, k, v = qkv.unbind(dim=1)
+    kh = k[seg_start:seg_end].transpose(0, 1).unsqueeze(0)
+    vh = v[seg_start:seg_end].transpose(0, 1).unsqueeze(0)
+    mask = None if perkey_bias is None else perkey_bias[seg_start:seg_end].to(qkv.dtype)[None, None, None, :]
+    qh = q[q_start:q_end].transpose(0, 1).unsqueeze(0)
+    return torch.nn.functional.scaled_dot_product_attention(qh, kh, vh, attn_mask=mask, scale=scale)[0].transpose(0, 1)
