@@ -49,7 +49,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "copy"], default=None,
+    ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "copy", "e2e"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -227,6 +228,45 @@ def bench_merge_unmerge(device, iters=200, warmup=20):
     }
 
 
+def bench_e2e(device, frames=32, depth=24, reps=5):
+    """End-to-end aggregator (random init, bf16): 24 frame + 24 global blocks, dim 1024, 16 heads x 64, MLP 4096,
+    32 frames of 518x518; 3x3 merge from block 4 onward at ratio 0.5 against the same model without merging."""
+    import torch
+    from come_amd.harness import AggregatorConfig, AlternatingAggregator, relative_l1
+    from come_amd.token_merger import CoMe_2D_TokenMerger
+
+    torch.manual_seed(0)
+    cfg = AggregatorConfig(depth=depth)
+    model = AlternatingAggregator(cfg).eval().to(device=device, dtype=torch.bfloat16)
+    images = torch.rand(1, frames, 3, 518, 518, generator=torch.Generator().manual_seed(0)).to(device)
+    merger = CoMe_2D_TokenMerger(cfg.specials, 3, 3, 0.5, allow_remainder=True)
+
+    def timed(m):
+        out = model(images, merger=m)                           # warm-up (allocator, GEMM heuristics)
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            out = model(images, merger=m)
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3)
+        return out, sorted(times)[len(times) // 2]
+
+    dense, dense_ms = timed(None)
+    merged, merged_ms = timed(merger)
+    mask = merged["merge_mask"].reshape(frames, 12, 12)
+    keep = torch.ones(frames, 37, 37, dtype=torch.bool, device=device)
+    keep[:, :36, :36] = ~mask.repeat_interleave(3, 1).repeat_interleave(3, 2)
+    keep_px = keep.repeat_interleave(14, 1).repeat_interleave(14, 2)[None, :, None]
+    return {"workload": f"VGGT-style aggregator, random init, bf16: {depth} frame + {depth} global blocks, dim 1024, "
+                        f"16 heads x 64, MLP 4096, S={frames} frames 518x518 ({dense['tokens_dense']} tokens); 3x3 merge "
+                        f"from block {cfg.merge_block} at r=0.5 ({merged['tokens_packed']} packed tokens)",
+            "merged_ms": round(merged_ms, 2), "unmerged_ms": round(dense_ms, 2),
+            "speedup": round(dense_ms / merged_ms, 3), "reps": reps, "statistic": "median wall time per forward",
+            "rel_l1_unmerged_windows": round(relative_l1(merged["maps"], dense["maps"], keep_px), 5),
+            "rel_l1_tolerance": 5e-2}
+
+
 # ------------------------------------------------------------------------------------------
 # host-CPU baseline (the reference's PyTorch path on the CPU), bounded sample
 # ------------------------------------------------------------------------------------------
@@ -307,7 +347,9 @@ def main():
     torch.cuda.set_device(device)
 
     if args.only:
-        if args.only == "copy":
+        if args.only == "e2e":
+            print(json.dumps({"only": "e2e", **bench_e2e(device, reps=max(1, args.steps))}))
+        elif args.only == "copy":
             # plain device copy of known size: the yardstick the HBM byte counters are scaled by
             nbytes = 256 << 20
             src = torch.empty(nbytes, dtype=torch.uint8, device=device).random_(0, 255)
@@ -361,6 +403,8 @@ def main():
     if not args.no_other:
         mw, other = bench_merge_unmerge(device)
         result["other"] = other
+    if not args.no_e2e:
+        result.setdefault("other", {})["e2e"] = bench_e2e(device)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_attention(w)
         if mw is not None:
