@@ -39,6 +39,8 @@ SIGNATURES = {
     "come_attn_varlen_fwd": (_int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64,
                                     _ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _f32,
                                     _ptr, _i64, _i64, _ptr, _ptr]),
+    "come_qk_norm_rope": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
+                                 _int, _ptr, _ptr, _ptr, _ptr, _f32, _ptr, _ptr, _ptr, _i64, _ptr]),
 }
 
 _lock = threading.Lock()

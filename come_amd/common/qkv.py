@@ -1,0 +1,96 @@
+"""Packed q/k preparation for the varlen attention: q/k LayerNorm + 2-D RoPE in one HIP kernel.
+
+Mirrors ``prepare_packed_self_attention_qkv`` of the reference
+(``src/accelerate/common/qkv.py:7-39``, inference branch ``:31-39``) and the parts of
+``RotaryPositionEmbedding2D`` it relies on (``src/thirdparty/vggt/layers/rope.py:62-117``:
+frequency tables with the angles rounded to the run dtype before cos / sin).  The packed tensor is
+updated in place, as in the reference; there is no out-of-place (autograd) branch.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+
+
+class RotaryPositionEmbedding2D:
+    """Holds the base frequency and caches the cos / sin tables ``[n_pos, head_dim // 4]``."""
+
+    def __init__(self, frequency: float = 100.0):
+        self.base_frequency = float(frequency)
+        self._cache: dict = {}
+
+    def tables(self, head_dim: int, n_pos: int, device, dtype):
+        key = (head_dim, n_pos, str(device), dtype)
+        if key not in self._cache:
+            half = head_dim // 2
+            exponents = torch.arange(0, half, 2, device=device).float() / half
+            inv_freq = 1.0 / (self.base_frequency ** exponents)
+            positions = torch.arange(n_pos, device=device, dtype=inv_freq.dtype)
+            angles = torch.einsum("i,j->ij", positions, inv_freq).to(dtype)
+            self._cache[key] = (angles.cos().to(dtype).contiguous(), angles.sin().to(dtype).contiguous())
+        return self._cache[key]
+
+
+_TABLES: dict[float, RotaryPositionEmbedding2D] = {}
+
+
+def _norm_params(norm):
+    """LayerNorm -> (apply, weight, bias, eps); Identity / None -> no normalisation."""
+    if norm is None or isinstance(norm, torch.nn.Identity):
+        return False, None, None, 0.0
+    if isinstance(norm, torch.nn.LayerNorm):
+        return True, norm.weight, norm.bias, float(norm.eps)
+    raise RuntimeError(f"q_norm / k_norm must be LayerNorm or Identity, got {type(norm).__name__}")
+
+
+def prepare_packed_self_attention_qkv(qkv: torch.Tensor, q_norm, k_norm, rope, pos: torch.Tensor | None,
+                                      run_dtype: torch.dtype, max_position: int | None = None) -> torch.Tensor:
+    """Normalises the packed q and k (``qkv [P, 3, H, D]``) and applies the 2-D RoPE, in place.
+
+    ``rope`` is an object with ``base_frequency`` (or ``None``), ``pos [P, 2]`` / ``[1, P, 2]`` integer
+    (y, x).  ``max_position`` (largest coordinate that can occur) avoids the device-to-host read of
+    ``pos.max()`` that sizes the frequency tables.
+    """
+    if torch.is_grad_enabled() and qkv.requires_grad:
+        raise RuntimeError("prepare_packed_self_attention_qkv is forward only (in place); run it under torch.no_grad()")
+    if not qkv.is_cuda:
+        raise RuntimeError("qkv must be on the GPU")
+    if qkv.dim() != 4 or qkv.shape[1] != 3:
+        raise RuntimeError("qkv must be [P, 3, H, D]")
+    if qkv.dtype != run_dtype or run_dtype not in (torch.bfloat16, torch.float16):
+        raise RuntimeError("qkv must be bf16 / fp16 and match run_dtype")
+    if qkv.stride(-1) != 1:
+        raise RuntimeError("qkv must have unit stride in the last dimension")
+    P, _, H, D = qkv.shape
+    apply_q, qw, qb, q_eps = _norm_params(q_norm)
+    apply_k, kw, kb, k_eps = _norm_params(k_norm)
+    if apply_q != apply_k or (apply_q and q_eps != k_eps):
+        raise RuntimeError("q_norm and k_norm must be the same kind of layer with the same eps")
+    use_rope = rope is not None and pos is not None
+    dev = qkv.device
+
+    def as_dtype(t):
+        return None if t is None else t.detach().to(device=dev, dtype=run_dtype).contiguous()
+
+    qw, qb, kw, kb = as_dtype(qw), as_dtype(qb), as_dtype(kw), as_dtype(kb)
+    positions = cos_t = sin_t = None
+    n_pos = 0
+    if use_rope:
+        positions = pos.reshape(-1, 2).to(device=dev, dtype=torch.int64).contiguous()
+        if positions.shape[0] != P:
+            raise RuntimeError(f"pos must hold one (y, x) pair per packed row ({P}), got {positions.shape[0]}")
+        n_pos = (int(positions.max().item()) if max_position is None else int(max_position)) + 1 if P > 0 else 1
+        if not isinstance(rope, RotaryPositionEmbedding2D):      # any object with a base frequency (e.g. the reference's)
+            rope = _TABLES.setdefault(float(rope.base_frequency), RotaryPositionEmbedding2D(float(rope.base_frequency)))
+        cos_t, sin_t = rope.tables(D, n_pos, dev, run_dtype)
+    q, k = qkv[:, 0], qkv[:, 1]
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(lib.come_qk_norm_rope(q.data_ptr(), k.data_ptr(), _lib.dtype_code(run_dtype),
+                                         q.stride(0), q.stride(1), k.stride(0), k.stride(1), P, H, D,
+                                         1 if apply_q else 0, _lib.ptr(qw), _lib.ptr(qb), _lib.ptr(kw), _lib.ptr(kb),
+                                         q_eps, _lib.ptr(positions), _lib.ptr(cos_t), _lib.ptr(sin_t), n_pos,
+                                         _lib.current_stream(dev)))
+    return qkv

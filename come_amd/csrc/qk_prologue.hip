@@ -1,0 +1,178 @@
+// Attention prologue on the packed q / k rows, in place: LayerNorm over the head dimension
+// followed by the 2-D rotary position embedding, one pass over memory.
+//
+// Layout: q and k are [total, n_heads, 64] views (unit stride inside a head) of the packed
+// projection output.  One lane owns 8 consecutive elements (16 bytes) of one head, so the
+// eight lanes of a head hold its 64 elements; reductions and the rotation partner
+// (element j <-> j +- 16 inside each 32-element half) are lane exchanges inside that group of
+// eight.  The first 32 elements of a head rotate with the y coordinate, the last 32 with x;
+// the angle of element j of a half is position * base^(-(j mod 16) / 16), looked up in
+// tables [n_pos, 16] that the caller builds in the tensor dtype.
+//
+// Rounding follows a chain of tensor operations in the storage dtype: the normalised value
+// is rounded once, each of the two products is rounded, and their sum is rounded.
+#include "come_common.h"
+
+namespace come {
+namespace {
+
+struct QkArgs {
+    void *ptr[2];                 // q, k
+    int64_t row_stride[2];        // elements
+    int64_t head_stride[2];
+    const void *gamma[2];         // [64] or nullptr
+    const void *beta[2];
+    int64_t total;
+    int n_heads;
+    int apply_norm;
+    float eps;
+    const int64_t *positions;     // [total, 2] (y, x) or nullptr: no rotation
+    const void *cos_table;        // [n_pos, 16]
+    const void *sin_table;
+    int64_t n_pos;
+};
+
+template <int DT>
+__device__ inline void round_to_dtype(float *f) {
+    const uint4 r = Vec16<DT>::pack(f);
+    Vec16<DT>::unpack(r, f);
+}
+
+__device__ inline float group8_sum(float v) {
+    v += __shfl_xor(v, 1);
+    v += __shfl_xor(v, 2);
+    v += __shfl_xor(v, 4);
+    return v;
+}
+
+template <int DT>
+__global__ void __launch_bounds__(256) qk_norm_rope_kernel(const QkArgs a) {
+    using V = Vec16<DT>;
+    const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const int lane8 = static_cast<int>(gid & 7);
+    const int64_t unit = gid >> 3;
+    const int head = static_cast<int>(unit % a.n_heads);
+    const int which = static_cast<int>((unit / a.n_heads) & 1);
+    const int64_t token = unit / (2 * a.n_heads);
+    if (token >= a.total) return;      // the eight lanes of a head leave together
+
+    uint4 *p = reinterpret_cast<uint4 *>(static_cast<char *>(a.ptr[which]) +
+                                         (token * a.row_stride[which] + head * a.head_stride[which]) * V::ELEM_BYTES) +
+               lane8;
+    float f[8];
+    V::unpack(*p, f);
+
+    if (a.apply_norm) {
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s += f[i];
+        const float mean = group8_sum(s) * (1.0f / 64.0f);
+        float q = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            f[i] -= mean;
+            q += f[i] * f[i];
+        }
+        const float rstd = rsqrtf(group8_sum(q) * (1.0f / 64.0f) + a.eps);
+        float g[8], b[8];
+        if (a.gamma[which] != nullptr) {
+            V::unpack(static_cast<const uint4 *>(a.gamma[which])[lane8], g);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) g[i] = 1.f;
+        }
+        if (a.beta[which] != nullptr) {
+            V::unpack(static_cast<const uint4 *>(a.beta[which])[lane8], b);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) b[i] = 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = f[i] * rstd * g[i] + b[i];
+        round_to_dtype<DT>(f);
+    }
+
+    if (a.positions != nullptr) {
+        // lanes 0-3 hold the y half, lanes 4-7 the x half; lanes {0,1} and {2,3} of a half are partners
+        int64_t pos = a.positions[token * 2 + (lane8 >> 2)];
+        pos = pos < 0 ? 0 : (pos >= a.n_pos ? a.n_pos - 1 : pos);
+        const int64_t entry = (pos * 16 + (lane8 & 1) * 8) * V::ELEM_BYTES;
+        float c[8], s[8], t[8];
+        V::unpack(*reinterpret_cast<const uint4 *>(static_cast<const char *>(a.cos_table) + entry), c);
+        V::unpack(*reinterpret_cast<const uint4 *>(static_cast<const char *>(a.sin_table) + entry), s);
+        const float sign = (lane8 & 2) ? 1.f : -1.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float partner = __shfl_xor(f[i], 2);
+            t[i] = sign * partner * s[i];
+            f[i] = f[i] * c[i];
+        }
+        round_to_dtype<DT>(t);
+        round_to_dtype<DT>(f);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] += t[i];
+    }
+    *p = V::pack(f);
+}
+
+}  // namespace
+}  // namespace come
+
+extern "C" int come_qk_norm_rope(void *q, void *k, int dtype,
+                                 int64_t q_row_stride, int64_t q_head_stride,
+                                 int64_t k_row_stride, int64_t k_head_stride,
+                                 int64_t total, int64_t n_heads, int64_t head_dim,
+                                 int apply_norm, const void *q_weight, const void *q_bias,
+                                 const void *k_weight, const void *k_bias, float eps,
+                                 const int64_t *positions, const void *cos_table, const void *sin_table,
+                                 int64_t n_pos, void *stream) {
+    using namespace come;
+    clear_error();
+    COME_REQUIRE(dtype == COME_BF16 || dtype == COME_F16, COME_ERR_UNSUPPORTED,
+                 "come_qk_norm_rope: dtype must be bf16 or fp16");
+    COME_REQUIRE(head_dim == 64, COME_ERR_UNSUPPORTED, "come_qk_norm_rope: only head_dim 64 is implemented (got %lld)",
+                 static_cast<long long>(head_dim));
+    COME_REQUIRE(total >= 0 && n_heads > 0 && n_heads < (1 << 20), COME_ERR_INVALID, "come_qk_norm_rope: bad sizes");
+    if (total == 0) return COME_OK;
+    COME_REQUIRE(q != nullptr && k != nullptr, COME_ERR_INVALID, "come_qk_norm_rope: null q / k");
+    const int64_t strides[4] = {q_row_stride, q_head_stride, k_row_stride, k_head_stride};
+    for (int64_t s : strides)
+        COME_REQUIRE(s >= 64 && s % 8 == 0, COME_ERR_INVALID,
+                     "come_qk_norm_rope: strides must be multiples of 8 elements and at least 64");
+    COME_REQUIRE(q_row_stride >= q_head_stride * (n_heads - 1) + 64 && k_row_stride >= k_head_stride * (n_heads - 1) + 64,
+                 COME_ERR_INVALID, "come_qk_norm_rope: heads of one row overlap the next row");
+    const void *aligned[] = {q, k, q_weight, q_bias, k_weight, k_bias, cos_table, sin_table};
+    for (const void *p : aligned)
+        COME_REQUIRE((reinterpret_cast<uintptr_t>(p) & 15) == 0, COME_ERR_INVALID,
+                     "come_qk_norm_rope: pointers must be 16-byte aligned");
+    COME_REQUIRE(eps >= 0.f, COME_ERR_INVALID, "come_qk_norm_rope: eps must be >= 0");
+    if (positions != nullptr)
+        COME_REQUIRE(cos_table != nullptr && sin_table != nullptr && n_pos > 0, COME_ERR_INVALID,
+                     "come_qk_norm_rope: positions need cos / sin tables with n_pos > 0");
+    if (!apply_norm && positions == nullptr) return COME_OK;
+
+    QkArgs a{};
+    a.ptr[0] = q; a.ptr[1] = k;
+    a.row_stride[0] = q_row_stride; a.row_stride[1] = k_row_stride;
+    a.head_stride[0] = q_head_stride; a.head_stride[1] = k_head_stride;
+    a.gamma[0] = q_weight; a.gamma[1] = k_weight;
+    a.beta[0] = q_bias; a.beta[1] = k_bias;
+    a.total = total;
+    a.n_heads = static_cast<int>(n_heads);
+    a.apply_norm = apply_norm;
+    a.eps = eps;
+    a.positions = positions;
+    a.cos_table = cos_table;
+    a.sin_table = sin_table;
+    a.n_pos = n_pos;
+    const int64_t threads = total * 2 * n_heads * 8;
+    const int64_t blocks = ceil_div(threads, 256);
+    COME_REQUIRE(blocks < (int64_t{1} << 31), COME_ERR_UNSUPPORTED, "come_qk_norm_rope: too many tokens for one launch");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == COME_BF16)
+        hipLaunchKernelGGL((qk_norm_rope_kernel<COME_BF16>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, a);
+    else
+        hipLaunchKernelGGL((qk_norm_rope_kernel<COME_F16>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, a);
+    COME_CHECK_LAUNCH("come_qk_norm_rope");
+    return COME_OK;
+}

@@ -13,9 +13,10 @@ camera / register tokens: first frame and other frames, LayerScale 0.01, RoPE ba
 
 The backbone the reference wraps (DINOv2 encoder, DPT heads, trained weights) is replaced by a
 14x14 patch-embedding convolution and a light dense head; weights are random.  All operators are
-injected: ``merger`` implements ``ITokenMerger`` and ``attention`` has the signature of
-``flash_attn_varlen_qkvpacked_func_w_perkey_bias``, so the same model runs on the HIP kernels (the
-default) or on any other implementation of the two interfaces.
+injected: ``merger`` implements ``ITokenMerger``, ``attention`` has the signature of
+``flash_attn_varlen_qkvpacked_func_w_perkey_bias`` and ``prologue`` that of
+``prepare_packed_self_attention_qkv`` (``src/accelerate/common/qkv.py:7-39``), so the same model runs on
+the HIP kernels (the default) or on any other implementation of the three interfaces.
 """
 
 from __future__ import annotations
@@ -60,34 +61,18 @@ def _default_attention(qkv, cu_seqlens, max_seqlen, perkey_bias, softmax_scale):
                                                           softmax_scale=softmax_scale)
 
 
+def _default_prologue(qkv, q_norm, k_norm, rope_base, pos, max_position):
+    from .common import RotaryPositionEmbedding2D, prepare_packed_self_attention_qkv
+
+    rope = _ROPES.setdefault(rope_base, RotaryPositionEmbedding2D(rope_base))
+    return prepare_packed_self_attention_qkv(qkv, q_norm, k_norm, rope, pos, qkv.dtype, max_position=max_position)
+
+
+_ROPES: dict = {}
+
+
 def _max_seqlen(cu_seqlens: torch.Tensor) -> int:
     return int((cu_seqlens[1:] - cu_seqlens[:-1]).max().item())
-
-
-class RopeTables:
-    """cos / sin of the 2-D rotary embedding for packed positions ``[P, 2]`` (y, x), computed once per forward
-    (``src/thirdparty/vggt/layers/rope.py:100-187``: angles rounded to the run dtype before cos / sin; the first half
-    of a head rotates with y, the second with x)."""
-
-    def __init__(self, positions: torch.Tensor, head_dim: int, base: float, dtype: torch.dtype):
-        half = head_dim // 2
-        exponents = torch.arange(0, half, 2, device=positions.device).float() / half
-        inv_freq = 1.0 / (base ** exponents)
-        n_pos = int(positions.max().item()) + 1
-        angles = torch.arange(n_pos, device=positions.device, dtype=torch.float32)[:, None] * inv_freq[None, :]
-        angles = torch.cat((angles.to(dtype), angles.to(dtype)), dim=-1)                 # [n_pos, half]
-        cos_t, sin_t = angles.cos().to(dtype), angles.sin().to(dtype)
-        y, x = positions[:, 0], positions[:, 1]
-        self.cos = torch.cat((cos_t[y], cos_t[x]), dim=-1)[:, None, :]                   # [P, 1, head_dim]
-        self.sin = torch.cat((sin_t[y], sin_t[x]), dim=-1)[:, None, :]
-        self.quarter = half // 2
-
-    def apply(self, t: torch.Tensor) -> torch.Tensor:
-        """``t [P, H, head_dim]`` -> rotated copy."""
-        P, H, D = t.shape
-        parts = t.view(P, H, 2, 2, self.quarter)
-        rotated = torch.stack((-parts[:, :, :, 1], parts[:, :, :, 0]), dim=3).view(P, H, D)
-        return t * self.cos + rotated * self.sin
 
 
 class JaggedBlock(nn.Module):
@@ -96,7 +81,7 @@ class JaggedBlock(nn.Module):
     def __init__(self, cfg: AggregatorConfig):
         super().__init__()
         C, D = cfg.dim, cfg.dim // cfg.heads
-        self.heads, self.head_dim = cfg.heads, D
+        self.heads, self.head_dim, self.rope_base = cfg.heads, D, cfg.rope_base
         self.norm1 = nn.LayerNorm(C)
         self.qkv = nn.Linear(C, 3 * C)
         self.q_norm, self.k_norm = nn.LayerNorm(D), nn.LayerNorm(D)
@@ -106,11 +91,10 @@ class JaggedBlock(nn.Module):
         self.fc1, self.fc2 = nn.Linear(C, cfg.mlp_dim), nn.Linear(cfg.mlp_dim, C)
         self.ls2 = nn.Parameter(torch.full((C,), cfg.layer_scale))
 
-    def forward(self, x, rope: RopeTables, cu_seqlens, max_seqlen, perkey_bias, attention) -> torch.Tensor:
+    def forward(self, x, pos, max_position, cu_seqlens, max_seqlen, perkey_bias, attention, prologue) -> torch.Tensor:
         P, C = x.shape
         qkv = self.qkv(self.norm1(x)).view(P, 3, self.heads, self.head_dim)
-        qkv[:, 0].copy_(rope.apply(self.q_norm(qkv[:, 0])))
-        qkv[:, 1].copy_(rope.apply(self.k_norm(qkv[:, 1])))
+        qkv = prologue(qkv, self.q_norm, self.k_norm, self.rope_base, pos, max_position)
         o = attention(qkv, cu_seqlens, max_seqlen, perkey_bias, self.head_dim ** -0.5)
         x = x + self.ls1 * self.proj(o.reshape(P, C).to(x.dtype))
         return x + self.ls2 * self.fc2(nn.functional.gelu(self.fc1(self.norm2(x))))
@@ -139,9 +123,12 @@ class AlternatingAggregator(nn.Module):
         """``images [B, S, 3, H, W]`` -> tokens ``[B, S, N, C]``, positions ``[B, S, N, 2]`` (y, x; specials 0,
         patches 1-based), grid ``(gh, gw)``."""
         B, S, _, H, W = images.shape
-        x = self.patch_embed(images.flatten(0, 1).to(self.patch_embed.weight.dtype))     # [B*S, C, gh, gw]
-        gh, gw = x.shape[-2:]
-        patches = x.flatten(2).transpose(1, 2)                                            # [B*S, gh*gw, C]
+        p = self.cfg.patch
+        gh, gw = H // p, W // p
+        # the stride-p convolution as one GEMM over unfolded patches (same weights, same arithmetic)
+        x = images.flatten(0, 1)[:, :, : gh * p, : gw * p].to(self.patch_embed.weight.dtype)
+        x = x.reshape(B * S, 3, gh, p, gw, p).permute(0, 2, 4, 1, 3, 5).reshape(B * S, gh * gw, 3 * p * p)
+        patches = nn.functional.linear(x, self.patch_embed.weight.flatten(1), self.patch_embed.bias)
 
         def first_and_others(tok):
             return torch.cat((tok[:, :1].expand(B, 1, -1, -1), tok[:, 1:].expand(B, S - 1, -1, -1)), dim=1).flatten(0, 1)
@@ -175,19 +162,21 @@ class AlternatingAggregator(nn.Module):
     # ---- forward --------------------------------------------------------------------------
     @torch.no_grad()
     def forward(self, images: torch.Tensor, merger: ITokenMerger | None = None,
-                attention: Callable | None = None) -> dict:
+                attention: Callable | None = None, prologue: Callable | None = None) -> dict:
         """Runs the aggregator.  ``merger = None``: every block on the dense token set (the unmerged baseline, same
         kernels with every count equal to 1 and no bias).  Otherwise blocks ``>= merge_block`` run on the packed
         tokens ``merger`` produces from the confidence predicted at ``merge_block``."""
         cfg = self.cfg
         attention = _default_attention if attention is None else attention
+        prologue = _default_prologue if prologue is None else prologue
         tokens, pos, (gh, gw) = self.embed(images)
         B, S, N, C = tokens.shape
         dev, dtype = tokens.device, tokens.dtype
         dense_offset = torch.arange(0, B * S + 1, device=dev, dtype=torch.int64) * N
 
+        max_position = max(gh, gw)                              # patch coordinates are 1-based, specials sit at 0
         state = dict(x=tokens.reshape(B * S * N, C), offset=dense_offset, weight=None, bias=None, ctx=None, stub=None,
-                     rope=RopeTables(pos.reshape(-1, 2), C // cfg.heads, cfg.rope_base, dtype))
+                     pos=pos.reshape(-1, 2).contiguous())
 
         def segments():
             frame = state["offset"].to(torch.int32)
@@ -205,12 +194,13 @@ class AlternatingAggregator(nn.Module):
                 merged, stub = merger.merge(ctx, state["x"].view(B, S, N, C))
                 merged_pos = merger.merge(ctx, pos.to(torch.bfloat16), stub=stub)[0].tokens.squeeze(0).long()
                 state.update(x=merged.tokens.squeeze(0), offset=merged.offset, weight=merged.weight, ctx=ctx, stub=stub,
-                             bias=merged.weight.float().log().to(dtype),
-                             rope=RopeTables(merged_pos, C // cfg.heads, cfg.rope_base, dtype))
+                             bias=merged.weight.float().log().to(dtype), pos=merged_pos)
                 (cu_f, max_f), (cu_g, max_g) = segments()
                 info.update(tokens_packed=int(merged.tokens.shape[1]), merge_mask=ctx[0] if isinstance(ctx, tuple) else None)
-            x_frame = self.frame_blocks[i](state["x"], state["rope"], cu_f, max_f, state["bias"], attention)
-            x_glob = self.global_blocks[i](x_frame, state["rope"], cu_g, max_g, state["bias"], attention)
+            x_frame = self.frame_blocks[i](state["x"], state["pos"], max_position, cu_f, max_f, state["bias"],
+                                           attention, prologue)
+            x_glob = self.global_blocks[i](x_frame, state["pos"], max_position, cu_g, max_g, state["bias"],
+                                           attention, prologue)
             state["x"] = x_glob
             if i in cfg.taps:
                 if state["ctx"] is not None:

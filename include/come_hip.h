@@ -167,6 +167,41 @@ int come_attn_varlen_fwd(const void *q, const void *k, const void *v, int dtype,
                          void *out, int64_t o_row_stride, int64_t o_head_stride,
                          float *lse, void *stream);
 
+/*
+ * come_qk_norm_rope — attention prologue, in place on the packed projection output:
+ * LayerNorm over the head dimension of every q and k head, then the 2-D rotary position
+ * embedding.
+ *
+ *   q, k      [total, n_heads, head_dim] views of `dtype` (COME_BF16 or COME_F16), unit stride
+ *             inside a head, *_row_stride / *_head_stride in elements; overwritten
+ *   apply_norm  0 = no normalisation; otherwise y = (x - mean) * rsqrt(var + eps) * weight + bias
+ *             over the head_dim elements of a head (biased variance, fp32 arithmetic, one
+ *             rounding to `dtype`); q_weight / q_bias / k_weight / k_bias are [head_dim] of
+ *             `dtype`, NULL = 1 resp. 0
+ *   positions [total, 2] int64 (y, x) per row, or NULL = no rotation.  The first half of a
+ *             head rotates with y, the second with x; inside a half h of H = head_dim / 2
+ *             elements, out[j] = h[j] cos[j mod H/2] - h[j + H/2] sin[j mod H/2] for j < H/2
+ *             and out[j] = h[j] cos[j mod H/2] + h[j - H/2] sin[j mod H/2] otherwise, products
+ *             and sum each rounded to `dtype`.
+ *   cos_table, sin_table  [n_pos, head_dim / 4] of `dtype`: cos / sin of
+ *             position * base^(-i / (head_dim / 4)); positions are clamped to [0, n_pos)
+ * Only head_dim == 64 is implemented.
+ *
+ * Stands in for the inference branch of prepare_packed_self_attention_qkv
+ * (src/accelerate/common/qkv.py:31-39): q_norm / k_norm of
+ * src/thirdparty/vggt/layers/attention.py:40-41 and RotaryPositionEmbedding2D.forward
+ * (src/thirdparty/vggt/layers/rope.py:100-187), which the reference runs as eight tensor
+ * passes over q and k.
+ */
+int come_qk_norm_rope(void *q, void *k, int dtype,
+                      int64_t q_row_stride, int64_t q_head_stride,
+                      int64_t k_row_stride, int64_t k_head_stride,
+                      int64_t total, int64_t n_heads, int64_t head_dim,
+                      int apply_norm, const void *q_weight, const void *q_bias,
+                      const void *k_weight, const void *k_bias, float eps,
+                      const int64_t *positions, const void *cos_table, const void *sin_table,
+                      int64_t n_pos, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -33,6 +33,12 @@ Pinning status of each function (what fixes its answers besides this text):
                                       the reference's tests; reductions to
                                       torch SDPA, key-duplication identity,
                                       logsumexp identity.
+  qk_norm_rope / rope_2d              layer_norm is the library routine; the
+                                      rotation is PARITY UNPINNED by the
+                                      reference's tests and pinned here by
+                                      closed forms (identity at 0, pair norms,
+                                      single-pair angle, relative-position
+                                      property of q.k).
 """
 
 from .jagged import JaggedTokens  # noqa: F401
@@ -52,3 +58,4 @@ from .attention import (  # noqa: F401
     biased_varlen_attention_sdpa_bf16,
     sdpa_bf16_chunk,
 )
+from .qk_prologue import qk_norm_rope, rope_2d, rope_tables  # noqa: F401

@@ -1,5 +1,5 @@
 """Oracle-backed operators for the end-to-end harness: the same two interfaces the HIP path
-implements (``ITokenMerger`` and the varlen attention callable), built on ``oracle/`` only."""
+implements (``ITokenMerger``, the varlen attention callable and the q/k prologue), built on ``oracle/`` only."""
 
 from __future__ import annotations
 
@@ -40,3 +40,9 @@ def oracle_attention(qkv, cu_seqlens, max_seqlen, perkey_bias, softmax_scale):
     out, _ = oracle.biased_varlen_attention(qkv.cpu(), cu_seqlens.cpu(), None if perkey_bias is None else perkey_bias.cpu(),
                                             softmax_scale)
     return out.to(device=qkv.device, dtype=qkv.dtype)
+
+
+def oracle_prologue(qkv, q_norm, k_norm, rope_base, pos, max_position):
+    out = oracle.qk_norm_rope(qkv.cpu(), q_norm.weight.cpu(), q_norm.bias.cpu(), k_norm.weight.cpu(), k_norm.bias.cpu(),
+                              q_norm.eps, pos.cpu(), rope_base)
+    return out.to(qkv.device)

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from come_amd.harness import AggregatorConfig, AlternatingAggregator, relative_l1
-from harness_oracle import OracleMerger, oracle_attention
+from harness_oracle import OracleMerger, oracle_attention, oracle_prologue
 
 pytestmark = pytest.mark.gpu
 
@@ -28,7 +28,7 @@ def test_kernel_path_matches_oracle_path():
     model = build(256, 4, 3, 1, (1, 2))
     images = torch.rand(1, 2, 3, 518, 518, generator=torch.Generator().manual_seed(3)).cuda()
     hip = model(images, merger=hip_merger(0.5))
-    ref = model(images, merger=OracleMerger(5, 3, 3, 0.5), attention=oracle_attention)
+    ref = model(images, merger=OracleMerger(5, 3, 3, 0.5), attention=oracle_attention, prologue=oracle_prologue)
     assert hip["tokens_packed"] == ref["tokens_packed"] == 1596
     assert torch.equal(hip["merge_mask"].cpu(), ref["merge_mask"])
     # stated tolerance for the kernel path against the oracle path of the same merged model
@@ -39,7 +39,7 @@ def test_unmerged_kernel_path_matches_oracle_path():
     model = build(256, 4, 2, 1, (0, 1))
     images = torch.rand(1, 2, 3, 518, 518, generator=torch.Generator().manual_seed(4)).cuda()
     hip = model(images, merger=None)
-    ref = model(images, merger=None, attention=oracle_attention)
+    ref = model(images, merger=None, attention=oracle_attention, prologue=oracle_prologue)
     assert relative_l1(hip["maps"], ref["maps"]) < 1e-2
 
 
