@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "copy", "e2e"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "copy", "e2e", "stress", "frame"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -147,13 +147,31 @@ def bench_attention(steps, warmup, device):
     return w, wall, ev_ms
 
 
-def merge_workload(device, ratio=0.5, sets=8):
+def jittered_frame_masks(conf, ratio, jitter, seed):
+    """Per-frame selection for the stress workload: frame f merges its ``round(r_f * M)`` lowest-confidence 3x3
+    windows with ``r_f = ratio + U(-jitter, jitter)`` (workload synthesis on the host side of the bench, torch)."""
+    import torch
+
+    frames, H, W = conf.shape
+    mh, mw = H // 3, W // 3
+    means = conf[:, : mh * 3, : mw * 3].reshape(frames, mh, 3, mw, 3).mean(dim=(2, 4)).reshape(frames, mh * mw)
+    g = torch.Generator().manual_seed(seed)
+    r = ratio + (torch.rand(frames, generator=g) * 2 - 1) * jitter
+    k = (r * mh * mw).round().long().clamp(0, mh * mw)
+    order = means.argsort(dim=1)
+    rank = torch.empty_like(order)
+    rank.scatter_(1, order, torch.arange(mh * mw).expand(frames, -1))
+    return rank < k[:, None]
+
+
+def merge_workload(device, ratio=0.5, sets=8, frames=16, H=37, W=37, jitter=None):
     """BASELINE merge microbench: 16 frames, 37x37 patches + 5 specials, C = 1024, bf16.  ``sets`` rotating
-    input / output buffer sets keep the working set (> 500 MB) out of the 256 MB Infinity Cache."""
+    input / output buffer sets keep the working set (> 500 MB) out of the 256 MB Infinity Cache.  With ``jitter``
+    the mask comes from ``jittered_frame_masks`` instead of the joint quantile selection."""
     import torch
     from come_amd import _lib
 
-    frames, H, W, S0, C = 16, 37, 37, 5, 1024
+    S0, C = 5, 1024
     N = S0 + H * W
     lib = _lib.load()
     conf = smooth_confidence(frames, H, W, seed=0).to(device)
@@ -167,9 +185,13 @@ def merge_workload(device, ratio=0.5, sets=8):
     prefix = torch.empty(frames, M, dtype=torch.int32, device=device)
     stream = _lib.current_stream(device)
 
+    if jitter is not None:
+        mask.copy_(jittered_frame_masks(conf.cpu(), ratio, jitter, seed=1).to(torch.uint8))
+
     def select_and_plan():
-        _lib.check(lib.come_select_windows(conf.data_ptr(), _lib.COME_F32, 1, frames, H, W, 3, 3, 0, ratio,
-                                           means.data_ptr(), mask.data_ptr(), None, 0, stream))
+        if jitter is None:
+            _lib.check(lib.come_select_windows(conf.data_ptr(), _lib.COME_F32, 1, frames, H, W, 3, 3, 0, ratio,
+                                               means.data_ptr(), mask.data_ptr(), None, 0, stream))
         _lib.check(lib.come_merge_plan(mask.data_ptr(), frames, M, S0, 9, tail, offsets.data_ptr(),
                                        prefix.data_ptr(), stream))
 
@@ -200,7 +222,8 @@ def merge_workload(device, ratio=0.5, sets=8):
     split_bytes = P * C * 2 + frames * N * 4 + frames * N * C * 2
     return dict(merge_only=merge_only, pipeline=pipeline, split_only=split_only, P=P, merge_bytes=merge_bytes,
                 split_bytes=split_bytes, frames=frames, N=N, C=C, ratio=ratio, tokens=tokens, conf=conf,
-                keep=(outs, restored, index_map, counts, mask, means, offsets, prefix))
+                counts=counts, offsets=offsets, outs=outs, restored=restored, index_map=index_map,
+                keep=(mask, means, prefix))
 
 
 def bench_merge_unmerge(device, iters=200, warmup=20):
@@ -226,6 +249,94 @@ def bench_merge_unmerge(device, iters=200, warmup=20):
                                  "unit": "GB/s", "frac": round(split_gbs / PEAK_HBM_GBS, 4),
                                  "traffic": TRAFFIC_BYTES["unmerge"]}},
     }
+
+
+def bench_merge_ratios(device, iters=200, warmup=20):
+    """The merge / unmerge microbenchmark at the other two ratios of the configuration."""
+    import torch
+
+    out = {}
+    for ratio in (0.25, 0.75):
+        w = merge_workload(device, ratio=ratio)
+        for _ in range(8):
+            w["merge_only"]()
+        _, m_ms = time_loop(w["merge_only"], iters, warmup)
+        _, s_ms = time_loop(w["split_only"], iters, warmup)
+        out["r%03d" % round(ratio * 100)] = {
+            "P": w["P"], "merge_us": round(m_ms / iters * 1e3, 2), "merge_bytes": w["merge_bytes"],
+            "merge_GBs": round(w["merge_bytes"] / (m_ms / iters * 1e-3) / 1e9, 1),
+            "merge_frac": round(w["merge_bytes"] / (m_ms / iters * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+            "unmerge_us": round(s_ms / iters * 1e3, 2), "unmerge_bytes": w["split_bytes"],
+            "unmerge_GBs": round(w["split_bytes"] / (s_ms / iters * 1e-3) / 1e9, 1),
+            "unmerge_frac": round(w["split_bytes"] / (s_ms / iters * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+        del w
+        torch.cuda.empty_cache()
+    return out
+
+
+def attention_case(device, lens, counts, steps, warmup, H=16, D=64):
+    """Times the biased attention on packed segments ``lens`` with per-key counts; returns (ms, TFLOP/s)."""
+    import torch
+    from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
+
+    P = sum(lens)
+    torch.manual_seed(1)
+    qkv = torch.randn(P, 3, H, D, device=device, dtype=torch.float32).bfloat16()
+    bias = counts.float().log().bfloat16().to(device)
+    bounds = [0]
+    for n in lens:
+        bounds.append(bounds[-1] + n)
+    cu = torch.tensor(bounds, dtype=torch.int32, device=device)
+    max_len = max(lens)
+    _, ms = time_loop(lambda: flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, max_len, perkey_bias=bias,
+                                                                             softmax_scale=0.125), steps, warmup)
+    flops = sum(4.0 * n * n * D * H for n in lens)
+    return ms / steps, flops / (ms / steps * 1e-3) / 1e12, flops
+
+
+def bench_frame_attention(device, w):
+    """Frame-mode attention of the headline workload's first sequence: 32 segments of about 798 tokens."""
+    import torch
+
+    counts = packed_counts(32, 144, 5, 73, 2304, torch.Generator().manual_seed(0))
+    # a frame ends where its counts add up to its 5 + 73 + 144 * 9 source tokens
+    ends = (counts.cumsum(0) % (5 + 73 + 144 * 9) == 0).nonzero().flatten() + 1
+    lens = torch.diff(ends, prepend=torch.zeros(1, dtype=ends.dtype)).tolist()
+    assert len(lens) == 32 and sum(lens) == counts.numel()
+    ms, tflops, flops = attention_case(device, lens, counts, steps=50, warmup=10)
+    return {"workload": "frame attention: 32 segments of %d..%d packed tokens (same tokens as the headline sequence 0)"
+                        % (min(lens), max(lens)), "us_per_call": round(ms * 1e3, 1), "value": round(tflops, 1),
+            "unit": "TFLOP/s", "algorithmic_flops": flops, "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
+
+
+def bench_stress(device):
+    """Long-sequence stress configuration at kernel level: 128 frames of 37x28 patches + 5 specials (133 248
+    tokens), 3x3 merge at ratio 0.75 with per-frame jitter +-0.1."""
+    import torch
+
+    w = merge_workload(device, ratio=0.75, sets=3, frames=128, H=37, W=28, jitter=0.1)
+    for _ in range(3):
+        w["merge_only"]()
+    _, m_ms = time_loop(w["merge_only"], 50, 10)
+    _, s_ms = time_loop(w["split_only"], 50, 10)
+    offsets = w["offsets"].cpu().tolist()
+    counts = w["counts"].cpu()
+    frame_lens = [b - a for a, b in zip(offsets[:-1], offsets[1:])]
+    res = {"workload": "stress: 128 frames 37x28+5 (133248 tokens), 3x3 merge r=0.75 +-0.1 per frame -> P=%d, "
+                       "frame segments %d..%d" % (w["P"], min(frame_lens), max(frame_lens)),
+           "merge_us": round(m_ms / 50 * 1e3, 1), "merge_bytes": w["merge_bytes"],
+           "merge_GBs": round(w["merge_bytes"] / (m_ms / 50 * 1e-3) / 1e9, 1),
+           "unmerge_us": round(s_ms / 50 * 1e3, 1), "unmerge_bytes": w["split_bytes"],
+           "unmerge_GBs": round(w["split_bytes"] / (s_ms / 50 * 1e-3) / 1e9, 1), "rotating_buffer_sets": 3}
+    P = w["P"]
+    del w
+    torch.cuda.empty_cache()
+    ms, tflops, flops = attention_case(device, frame_lens, counts, steps=20, warmup=5)
+    res["frame_attention"] = {"us_per_call": round(ms * 1e3, 1), "TFLOPs": round(tflops, 1), "algorithmic_flops": flops}
+    ms, tflops, flops = attention_case(device, [P], counts, steps=5, warmup=2)
+    res["global_attention"] = {"ms_per_call": round(ms, 3), "TFLOPs": round(tflops, 1), "algorithmic_flops": flops,
+                               "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
+    return res
 
 
 def bench_e2e(device, frames=32, depth=24, reps=5):
@@ -347,7 +458,11 @@ def main():
     torch.cuda.set_device(device)
 
     if args.only:
-        if args.only == "e2e":
+        if args.only == "stress":
+            print(json.dumps({"only": "stress", **bench_stress(device)}))
+        elif args.only == "frame":
+            print(json.dumps({"only": "frame", **bench_frame_attention(device, None)}))
+        elif args.only == "e2e":
             print(json.dumps({"only": "e2e", **bench_e2e(device, reps=max(1, args.steps))}))
         elif args.only == "copy":
             # plain device copy of known size: the yardstick the HBM byte counters are scaled by
@@ -403,6 +518,9 @@ def main():
     if not args.no_other:
         mw, other = bench_merge_unmerge(device)
         result["other"] = other
+        other["merge_other_ratios"] = bench_merge_ratios(device)
+        other["frame_attention"] = bench_frame_attention(device, w)
+        other["stress"] = bench_stress(device)
     if not args.no_e2e:
         result.setdefault("other", {})["e2e"] = bench_e2e(device)
     if not args.no_cpu_baseline:

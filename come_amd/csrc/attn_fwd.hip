@@ -50,7 +50,7 @@ struct AttnArgs {
     const int32_t *cu;
     int64_t q_rs, q_hs, k_rs, k_hs, v_rs, v_hs, o_rs, o_hs;
     int64_t total;
-    int n_heads, n_mblocks;
+    int n_heads, n_mblocks, n_units;
     float scale, scale_log2, inv_scale;
 };
 
@@ -101,6 +101,20 @@ __device__ inline s16x4 lds_read_tr(const uint16_t *p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(p));
 }
 
+// Which (segment, head, query block) a workgroup computes.  Workgroup i is dispatched to XCD
+// i % 8, each XCD with its own L2: the query blocks of one (segment, head) unit run back to back
+// on one XCD and share that unit's K/V there, and units are dealt to the XCDs round-robin so that
+// segments of different lengths spread evenly.  The grid is padded to 8 * ceil(units / 8) units.
+__device__ inline bool locate_block(const AttnArgs &a, int &mblk, int &head, int &seq) {
+    const int xcd = blockIdx.x & 7;
+    const int local = blockIdx.x >> 3;
+    const int unit = xcd + 8 * (local / a.n_mblocks);
+    mblk = local % a.n_mblocks;
+    head = unit % a.n_heads;
+    seq = unit / a.n_heads;
+    return unit < a.n_units;
+}
+
 template <int DT, int QT>
 __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnArgs a) {
     using E = Elem<DT>;
@@ -108,16 +122,8 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnArgs a) {
     __shared__ __attribute__((aligned(16))) uint16_t lds_k[2][kBlockN * kKPitch];
     __shared__ __attribute__((aligned(16))) uint16_t lds_v[2][kBlockN * kVPitch];
 
-    // ---- which (segment, head, query block): consecutive blocks of one (segment, head)
-    //      run on the same XCD (workgroup i is dispatched to XCD i % 8) and share K/V in its L2
-    const int n_wg = gridDim.x;
-    int wid = blockIdx.x;
-    const int per_xcd = n_wg >> 3;
-    if (wid < (per_xcd << 3)) wid = (wid & 7) * per_xcd + (wid >> 3);
-    const int mblk = wid % a.n_mblocks;
-    const int rest = wid / a.n_mblocks;
-    const int head = rest % a.n_heads;
-    const int seq = rest / a.n_heads;
+    int mblk, head, seq;
+    if (!locate_block(a, mblk, head, seq)) return;
     const int seq_start = a.cu[seq];
     const int L = a.cu[seq + 1] - seq_start;
     const int q0 = mblk * kBlockM;
@@ -365,16 +371,8 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
     __shared__ __attribute__((aligned(16))) uint16_t lds_b[kStages][kBlockN * kBiasPitch];
     __shared__ __attribute__((aligned(256))) uint32_t lds_braw[kStages][kBlockN];   // raw bias words as loaded
 
-    // consecutive query blocks of one (segment, head) run on the same XCD (workgroup i is
-    // dispatched to XCD i % 8) and share K/V in its L2
-    const int n_wg = gridDim.x;
-    int wid = blockIdx.x;
-    const int per_xcd = n_wg >> 3;
-    if (wid < (per_xcd << 3)) wid = (wid & 7) * per_xcd + (wid >> 3);
-    const int mblk = wid % a.n_mblocks;
-    const int rest = wid / a.n_mblocks;
-    const int head = rest % a.n_heads;
-    const int seq = rest / a.n_heads;
+    int mblk, head, seq;
+    if (!locate_block(a, mblk, head, seq)) return;
     const int seq_start = a.cu[seq];
     const int L = a.cu[seq + 1] - seq_start;
     const int q0 = mblk * kBlockM;
@@ -900,7 +898,8 @@ extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v,
     a.scale = softmax_scale;
     a.scale_log2 = softmax_scale * 1.4426950408889634f;
     a.inv_scale = 1.0f / softmax_scale;
-    const int64_t n_wg = n_seq * n_heads * a.n_mblocks;
+    a.n_units = static_cast<int>(n_seq * n_heads);
+    const int64_t n_wg = ceil_div(n_seq * n_heads, 8) * 8 * a.n_mblocks;
     COME_REQUIRE(n_wg < (1ll << 31), COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: grid too large");
     const dim3 grid(static_cast<unsigned>(n_wg)), block(kThreads);
     hipStream_t s = static_cast<hipStream_t>(stream);
