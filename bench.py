@@ -339,6 +339,20 @@ def bench_stress(device):
     return res
 
 
+def bench_gemm_reference(device):
+    """Library bf16 GEMM (8192^3, N(0,1) operands, torch.matmul -> hipBLASLt) in the same run: what the matrix
+    cores of this box sustain on data of the same kind, next to the nominal 2.5 PFLOP/s used for ``frac``."""
+    import torch
+
+    torch.manual_seed(0)
+    a = torch.randn(8192, 8192, device=device).bfloat16()
+    b = torch.randn(8192, 8192, device=device).bfloat16()
+    _, ms = time_loop(lambda: a @ b, 20, 5)
+    tflops = 2.0 * 8192 ** 3 / (ms / 20 * 1e-3) / 1e12
+    return {"workload": "torch.matmul bf16 8192x8192x8192, N(0,1) operands", "value": round(tflops, 1), "unit": "TFLOP/s",
+            "frac_of_nominal_peak": round(tflops / PEAK_BF16_TFLOPS, 4)}
+
+
 def bench_e2e(device, frames=32, depth=24, reps=5):
     """End-to-end aggregator (random init, bf16): 24 frame + 24 global blocks, dim 1024, 16 heads x 64, MLP 4096,
     32 frames of 518x518; 3x3 merge from block 4 onward at ratio 0.5 against the same model without merging."""
@@ -518,6 +532,7 @@ def main():
     if not args.no_other:
         mw, other = bench_merge_unmerge(device)
         result["other"] = other
+        other["library_gemm_reference"] = bench_gemm_reference(device)
         other["merge_other_ratios"] = bench_merge_ratios(device)
         other["frame_attention"] = bench_frame_attention(device, w)
         other["stress"] = bench_stress(device)
