@@ -1,10 +1,10 @@
 // Window confidence means and lowest-confidence window selection for gfx950.
 //
 // One workgroup per batch element: it reduces every full window of that element's
-// frames to its mean, finds the two order statistics that torch.quantile's linear
-// interpolation needs with an exact 4 x 8-bit radix select over the float bit
-// patterns, forms the threshold in fp32 and writes the strict "mean < threshold"
-// mask.  The data is tiny (thousands of means), so the kernel is latency bound; it
+// frames to its mean (kept in registers), finds the lower of the two order statistics
+// that torch.quantile's linear interpolation needs with an exact 4 x 8-bit radix select
+// over the float bit patterns and its upper neighbour with one more reduction, forms the
+// threshold in fp32 and writes the strict "mean < threshold" mask.  The data is tiny (thousands of means), so the kernel is latency bound; it
 // exists to keep the selection on the device and bit-exact.
 #include "come_common.h"
 
@@ -24,18 +24,32 @@ __device__ inline float key_to_float(uint32_t k) {
     return __uint_as_float(u);
 }
 
-// k-th smallest (0-based) of vals[0..n); all threads of the workgroup call it and
-// all receive the answer.  hist: 256 counters, ctl: 2 words of LDS.
-__device__ float radix_select(const float *vals, int n, int k, uint32_t *hist, uint32_t *ctl) {
+constexpr int kKeysPerThread = 8;      // means kept in registers up to 8 * 1024 per batch element
+
+// k-th smallest (0-based) of the n values the workgroup holds: thread t owns values t, t + 1024, ...
+// either in mine[] (n <= 8192) or in vals[] (global).  All threads call it and all receive the answer.
+// hist: 256 counters, ctl: 2 words of LDS.
+__device__ float radix_select(const float *vals, const float *mine, bool in_regs, int n, int k, uint32_t *hist,
+                              uint32_t *ctl) {
     uint32_t prefix = 0, fixed = 0;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     for (int shift = 24; shift >= 0; shift -= 8) {
         if (threadIdx.x < 256) hist[threadIdx.x] = 0;
         __syncthreads();
-        for (int i = threadIdx.x; i < n; i += blockDim.x) {
-            const uint32_t key = ordered_key(vals[i]);
-            if ((key & fixed) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+        if (in_regs) {
+#pragma unroll
+            for (int r = 0; r < kKeysPerThread; ++r) {
+                if (static_cast<int>(threadIdx.x) + r * kSelectThreads < n) {
+                    const uint32_t key = ordered_key(mine[r]);
+                    if ((key & fixed) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+                }
+            }
+        } else {
+            for (int i = threadIdx.x; i < n; i += blockDim.x) {
+                const uint32_t key = ordered_key(vals[i]);
+                if ((key & fixed) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+            }
         }
         __syncthreads();
         if (wave == 0) {
@@ -69,9 +83,32 @@ __device__ float radix_select(const float *vals, int n, int k, uint32_t *hist, u
         prefix |= ctl[0] << shift;
         fixed |= 255u << shift;
         k = static_cast<int>(ctl[1]);
-        __syncthreads();
     }
+    __syncthreads();                       // ctl and hist are free again
     return key_to_float(prefix);
+}
+
+// Workgroup-wide sum (every thread receives it).  red: 17 floats of LDS.
+__device__ float block_sum(float v, float *red) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    if (wave == 0) {
+        float t = lane < kSelectThreads / 64 ? red[lane] : 0.f;
+#pragma unroll
+        for (int d = 8; d >= 1; d >>= 1) t += __shfl_xor(t, d);
+        if (lane == 0) red[16] = t;
+    }
+    __syncthreads();
+    return red[16];
+}
+
+template <int DT> __device__ inline float round_dt(float x) {
+    if (DT == COME_BF16) return __uint_as_float(pack2_bf16(x, 0.f) << 16);
+    return x;
 }
 
 template <int DT>
@@ -81,6 +118,7 @@ __global__ __launch_bounds__(kSelectThreads) void select_windows_kernel(
     using V = Vec16<DT>;
     __shared__ uint32_t hist[256];
     __shared__ uint32_t ctl[2];
+    __shared__ float red[17];
 
     const int mh = H / gh, mw = W / gw;
     const int M = mh * mw;
@@ -88,10 +126,33 @@ __global__ __launch_bounds__(kSelectThreads) void select_windows_kernel(
     const int64_t batch_first = static_cast<int64_t>(blockIdx.x) * n;
     float *my_means = means + batch_first;
     uint8_t *my_mask = mask + batch_first;
+    const bool in_regs = n <= kKeysPerThread * kSelectThreads;
+
+    // 0. normalised-score mode: z = (x - mean) / (std + 1e-3) over all positions of the batch element,
+    //    every tensor operation of that chain rounded to the confidence dtype (unbiased std)
+    float z_mean = 0.f, z_denom = 1.f;
+    if (mode == 2) {
+        const int64_t T = static_cast<int64_t>(frames) * H * W;
+        const int64_t first = static_cast<int64_t>(blockIdx.x) * T;
+        float acc = 0.f;
+        for (int64_t i = threadIdx.x; i < T; i += blockDim.x) acc += V::load1(conf, first + i);
+        const float mean32 = block_sum(acc, red) / static_cast<float>(T);
+        acc = 0.f;
+        for (int64_t i = threadIdx.x; i < T; i += blockDim.x) {
+            const float d = V::load1(conf, first + i) - mean32;
+            acc += d * d;
+        }
+        const float var = block_sum(acc, red) / static_cast<float>(T > 1 ? T - 1 : 1);
+        z_mean = round_dt<DT>(mean32);
+        z_denom = round_dt<DT>(round_dt<DT>(sqrtf(var)) + 1e-3f);
+    }
 
     // 1. window means: fp32 running sum in window row-major order, one division,
     //    rounded to the confidence dtype and widened back to fp32
-    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float mine[kKeysPerThread];
+#pragma unroll
+    for (int r = 0; r < kKeysPerThread; ++r) mine[r] = 0.f;
+    auto window_mean = [&](int i) {
         const int f = i / M;
         const int m = i - f * M;
         const int wy = m / mw;
@@ -100,25 +161,70 @@ __global__ __launch_bounds__(kSelectThreads) void select_windows_kernel(
                              static_cast<int64_t>(wy * gh) * W + wx * gw;
         float acc = 0.f;
         for (int dy = 0; dy < gh; ++dy)
-            for (int dx = 0; dx < gw; ++dx) acc = __fadd_rn(acc, V::load1(conf, base + static_cast<int64_t>(dy) * W + dx));
-        float mean = __fdiv_rn(acc, static_cast<float>(gh * gw));
-        if (DT == COME_BF16) mean = __uint_as_float(pack2_bf16(mean, 0.f) << 16);
-        my_means[i] = mean;
+            for (int dx = 0; dx < gw; ++dx) {
+                float x = V::load1(conf, base + static_cast<int64_t>(dy) * W + dx);
+                if (mode == 2) x = round_dt<DT>(__fdiv_rn(round_dt<DT>(__fsub_rn(x, z_mean)), z_denom));
+                acc = __fadd_rn(acc, x);
+            }
+        return round_dt<DT>(__fdiv_rn(acc, static_cast<float>(gh * gw)));
+    };
+    if (in_regs) {
+#pragma unroll
+        for (int r = 0; r < kKeysPerThread; ++r) {
+            const int i = static_cast<int>(threadIdx.x) + r * kSelectThreads;
+            if (i < n) {
+                mine[r] = window_mean(i);
+                my_means[i] = mine[r];
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < n; i += blockDim.x) my_means[i] = window_mean(i);
+        __syncthreads();
     }
-    __syncthreads();
 
-    // 2. threshold
+    // 2. threshold.  Ranking: the two neighbouring order statistics of torch.quantile's linear interpolation;
+    //    the upper one is either the same value again (duplicates) or the smallest value above the lower one.
     float cut = threshold;
     if (mode == 0) {
-        const float a = radix_select(my_means, n, rank_lo, hist, ctl);
-        const float b = rank_hi == rank_lo ? a : radix_select(my_means, n, rank_hi, hist, ctl);
+        const float a = radix_select(my_means, mine, in_regs, n, rank_lo, hist, ctl);
+        float b = a;
+        if (rank_hi != rank_lo) {
+            float le = 0.f;                                   // exact in fp32: n < 2^24
+            uint32_t above = 0xffffffffu;                     // ordered key of the smallest value > a
+            const uint32_t key_a = ordered_key(a);
+            auto visit = [&](float x) {
+                const uint32_t key = ordered_key(x);
+                if (key <= key_a) le += 1.f;
+                else above = min(above, key);
+            };
+            if (in_regs) {
+#pragma unroll
+                for (int r = 0; r < kKeysPerThread; ++r)
+                    if (static_cast<int>(threadIdx.x) + r * kSelectThreads < n) visit(mine[r]);
+            } else {
+                for (int i = threadIdx.x; i < n; i += blockDim.x) visit(my_means[i]);
+            }
+            if (threadIdx.x == 0) ctl[0] = 0xffffffffu;
+            const float count_le = block_sum(le, red);       // its barriers also publish ctl[0]
+            atomicMin(&ctl[0], above);
+            __syncthreads();
+            if (count_le <= static_cast<float>(rank_hi)) b = key_to_float(ctl[0]);
+        }
         const float diff = __fsub_rn(b, a);
         cut = frac < 0.5f ? __fadd_rn(a, __fmul_rn(frac, diff))
                           : __fsub_rn(b, __fmul_rn(diff, __fsub_rn(1.0f, frac)));
     }
 
     // 3. strict comparison
-    for (int i = threadIdx.x; i < n; i += blockDim.x) my_mask[i] = my_means[i] < cut ? 1 : 0;
+    if (in_regs) {
+#pragma unroll
+        for (int r = 0; r < kKeysPerThread; ++r) {
+            const int i = static_cast<int>(threadIdx.x) + r * kSelectThreads;
+            if (i < n) my_mask[i] = mine[r] < cut ? 1 : 0;
+        }
+    } else {
+        for (int i = threadIdx.x; i < n; i += blockDim.x) my_mask[i] = my_means[i] < cut ? 1 : 0;
+    }
 }
 
 }  // namespace
@@ -144,7 +250,7 @@ extern "C" int come_select_windows(const void *conf, int dtype, int64_t batch, i
                  "come_select_windows: negative size");
     COME_REQUIRE(group_h > 0 && group_w > 0, COME_ERR_INVALID,
                  "come_select_windows: group_h and group_w must be > 0");
-    COME_REQUIRE(mode == 0 || mode == 1, COME_ERR_UNSUPPORTED, "come_select_windows: unknown mode %d", mode);
+    COME_REQUIRE(mode >= 0 && mode <= 2, COME_ERR_UNSUPPORTED, "come_select_windows: unknown mode %d", mode);
     if (mode == 0)
         COME_REQUIRE(threshold >= 0.f && threshold <= 1.f, COME_ERR_INVALID,
                      "come_select_windows: ranking mode requires threshold in [0, 1], got %g", (double)threshold);

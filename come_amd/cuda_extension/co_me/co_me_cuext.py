@@ -124,7 +124,7 @@ def co_me_token_merge_2d_cuda(tokens: torch.Tensor, start_index: int, group_h: i
                        index_dtype, count_dtype)
 
 
-_MODES = {"pairwise-rank": 0, "abs_mse": 1}
+_MODES = {"pairwise-rank": 0, "abs_mse": 1, "mse": 2}
 
 
 def co_me_select_windows(conf: torch.Tensor, batch: int, group_h: int, group_w: int, threshold: float,

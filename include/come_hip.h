@@ -121,13 +121,17 @@ int come_token_split(const void *merged, int dtype, int64_t merged_rows, int64_t
  *                mask = mean < quantile(float(mean), threshold) with torch.quantile's
  *                linear interpolation;
  *            1 = absolute: mask = mean < threshold
+ *            2 = normalised: the confidence of a batch element is first turned into
+ *                z = (x - mean) / (std + 1e-3) over all its positions (unbiased std, every
+ *                step rounded to `dtype`), then mask = window mean of z < threshold
  *   means_f32 [batch * frames, windows] float out (the means, rounded to `dtype` first);
  *            may be NULL
  *   merge_mask [batch * frames, windows] bytes out (1 = merge)
  *   work     device scratch of at least come_select_work_bytes(...) bytes
  *
  * Stands in for the window-mean + torch.quantile + compare sequence of
- * _CoMe_2D_Base.build_ctx (src/accelerate/token_merger/co_me_2d.py:268-298).
+ * _CoMe_2D_Base.build_ctx (src/accelerate/token_merger/co_me_2d.py:268-298; mode 2:
+ * :275-283).
  */
 int come_select_windows(const void *conf, int dtype, int64_t batch, int64_t frames,
                         int64_t grid_h, int64_t grid_w, int64_t group_h, int64_t group_w,

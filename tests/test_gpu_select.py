@@ -76,6 +76,40 @@ def test_negative_values_and_absolute_mode():
     assert torch.equal(mask.cpu(), oracle.select_lowest_confidence(conf, 1, 3, 3, 0.1, mode="abs_mse"))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("batch,frames,H,W", [(1, 4, 12, 12), (2, 8, 37, 37), (1, 32, 37, 28)])
+def test_normalised_score_mode(batch, frames, H, W, dtype):
+    """z-score mode (not exercised by any test of the reference: parity unpinned there).  The mean and the
+    standard deviation are long fp32 reductions whose last bit depends on the summation order, so the window
+    means may differ from the CPU oracle's by a rounding step of the confidence dtype; the mask is compared
+    bit for bit on every window whose oracle mean is further from the threshold than that, and those must be
+    nearly all windows."""
+    g = torch.Generator().manual_seed(batch * 100 + frames)
+    conf = (torch.rand(batch * frames, H, W, generator=g) * 3 + 1).to(dtype)
+    thr = -0.1
+    mask, means = co_me_cuext.co_me_select_windows(conf.to(DEV), batch, 3, 3, thr, mode="mse", return_means=True)
+    want = oracle.select_lowest_confidence(conf, batch, 3, 3, thr, mode="mse")
+    flat = conf.reshape(batch, -1)
+    z = (flat - flat.mean(dim=-1, keepdim=True)) / (flat.std(dim=-1, keepdim=True) + 1e-3)
+    want_means = oracle.window_confidence_means(z.reshape(-1, H, W), 3, 3).float()
+    step = 2.0 ** -6 if dtype == torch.bfloat16 else 1e-5
+    torch.testing.assert_close(means.cpu(), want_means, atol=step, rtol=0)
+    clear = (want_means - thr).abs() > step
+    assert float(clear.float().mean()) > 0.9
+    assert torch.equal(mask.cpu()[clear], want[clear])
+    assert 0 < int(mask.sum()) < mask.numel()
+
+
+def test_large_window_count_uses_the_global_path():
+    # more than 8192 windows per batch element: the means no longer fit the per-thread registers
+    conf = torch.rand(40, 45, 45, generator=torch.Generator().manual_seed(7))     # 40 * 225 = 9000 windows
+    for ratio in (0.3, 0.62):
+        mask = co_me_cuext.co_me_select_windows(conf.to(DEV), 1, 3, 3, ratio)
+        gpu_means = co_me_cuext.co_me_select_windows(conf.to(DEV), 1, 3, 3, ratio, return_means=True)[1].cpu()
+        cut = torch.quantile(gpu_means.reshape(1, -1), ratio, dim=-1, keepdim=True)
+        assert torch.equal(mask.cpu().reshape(1, -1), gpu_means.reshape(1, -1) < cut)
+
+
 @pytest.mark.parametrize("ratio", [0.25, 0.5, 0.75])
 def test_fused_select_merge_c2(ratio):
     B, S, H, W, C, S0 = 1, 16, 37, 37, 1024, 5
