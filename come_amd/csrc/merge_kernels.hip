@@ -26,6 +26,22 @@ __device__ inline void st16_stream(uint4 *p, const uint4 &v) {
     __builtin_nontemporal_store(w, reinterpret_cast<u32x4_t *>(p));
 }
 
+// x / d for 0 <= x < 2^31 as one 32 x 32 -> 64 bit multiply and a shift (mul = ceil(2^shift / d),
+// shift = 31 + ceil(log2 d)); the index arithmetic of the 16-byte kernels runs on these instead of the
+// compiler's division sequences, which sit in front of every thread's first load
+struct FastDiv {
+    uint32_t mul, shift;
+};
+inline FastDiv make_fastdiv(int64_t d) {
+    uint32_t s = 0;
+    while ((int64_t{1} << s) < d) ++s;
+    const uint64_t pow = uint64_t{1} << (31 + s);
+    return FastDiv{static_cast<uint32_t>((pow + static_cast<uint64_t>(d) - 1) / static_cast<uint64_t>(d)), 31 + s};
+}
+__device__ inline uint32_t fast_div(uint32_t x, const FastDiv &f) {
+    return static_cast<uint32_t>((static_cast<uint64_t>(x) * f.mul) >> f.shift);
+}
+
 struct MergeGeom {
     int rows, n_tok, start, groups;
     int gh, gw, G;          // window shape, tokens per window
@@ -50,6 +66,7 @@ struct MergeArgs {
     int64_t group_blocks;    // blocks that own group items
     int64_t single_items;    // rows * (start + tail) * chunks
     int chunks;              // 16-byte chunks per token row (vector kernel) / chans (scalar kernel)
+    FastDiv by_chunks, by_groups, by_mw, by_per_row, by_side;   // 16-byte kernels only
 };
 
 __device__ inline void note_row(const MergeArgs &a, int64_t src_flat, int64_t dst) {
@@ -68,6 +85,16 @@ __device__ inline int leftover_position(const MergeGeom &g, int r) {
     const int upper = g.cov_h * side;
     if (r < upper) {
         const int y = r / side;
+        return y * g.W + g.cov_w + (r - y * side);
+    }
+    return g.cov_h * g.W + (r - upper);
+}
+
+__device__ inline int leftover_position_fast(const MergeGeom &g, const FastDiv &by_side, int r) {
+    const int side = g.W - g.cov_w;
+    const int upper = g.cov_h * side;
+    if (r < upper) {
+        const int y = static_cast<int>(fast_div(static_cast<uint32_t>(r), by_side));
         return y * g.W + g.cov_w + (r - y * side);
     }
     return g.cov_h * g.W + (r - upper);
@@ -131,13 +158,13 @@ __global__ __launch_bounds__(kThreads) void merge_vec_kernel(const MergeArgs a) 
     const int chunks = a.chunks;
 
     if (static_cast<int64_t>(blockIdx.x) < a.group_blocks) {
-        const int64_t id = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+        const uint32_t id = blockIdx.x * kThreads + threadIdx.x;     // item counts stay below 2^31 (checked by the host)
         if (id >= a.group_items) return;
-        const int64_t gm = id / chunks;                     // flat (row, window)
+        const uint32_t gm = fast_div(id, a.by_chunks);      // flat (row, window)
         const int chunk = static_cast<int>(id - gm * chunks);
-        const int b = static_cast<int>(gm / g.groups);
-        const int m = static_cast<int>(gm - static_cast<int64_t>(b) * g.groups);
-        const int wy = m / g.mw;
+        const int b = static_cast<int>(fast_div(gm, a.by_groups));
+        const int m = static_cast<int>(gm) - b * g.groups;
+        const int wy = static_cast<int>(fast_div(m, a.by_mw));
         const int wx = m - wy * g.mw;
         const bool merged = a.mask[gm] != 0;
         const int64_t row0 = static_cast<int64_t>(a.offsets[b]) + g.start + a.prefix[gm];
@@ -212,13 +239,13 @@ __global__ __launch_bounds__(kThreads) void merge_vec_kernel(const MergeArgs a) 
     }
 
     // copied tokens: specials in front, leftover grid positions behind the windows
-    const int64_t id = (static_cast<int64_t>(blockIdx.x) - a.group_blocks) * kThreads + threadIdx.x;
+    const uint32_t id = (blockIdx.x - static_cast<uint32_t>(a.group_blocks)) * kThreads + threadIdx.x;
     if (id >= a.single_items) return;
     const int per_row = g.start + g.tail;
-    const int64_t t = id / chunks;
+    const uint32_t t = fast_div(id, a.by_chunks);
     const int chunk = static_cast<int>(id - t * chunks);
-    const int b = static_cast<int>(t / per_row);
-    const int j = static_cast<int>(t - static_cast<int64_t>(b) * per_row);
+    const int b = static_cast<int>(fast_div(t, a.by_per_row));
+    const int j = static_cast<int>(t) - b * per_row;
     int tok;
     int64_t row;
     if (j < g.start) {
@@ -226,7 +253,7 @@ __global__ __launch_bounds__(kThreads) void merge_vec_kernel(const MergeArgs a) 
         row = static_cast<int64_t>(a.offsets[b]) + j;
     } else {
         const int r = j - g.start;
-        tok = g.start + leftover_position(g, r);
+        tok = g.start + leftover_position_fast(g, a.by_side, r);
         row = static_cast<int64_t>(a.offsets[b + 1]) - g.tail + r;
     }
     const int64_t flat = static_cast<int64_t>(b) * g.n_tok + tok;
@@ -316,12 +343,13 @@ constexpr int kSplitRows = 4;      // output rows per thread (independent loads 
 template <typename IndexT>
 __global__ __launch_bounds__(kThreads) void split_vec_kernel(const uint4 *__restrict__ merged, int64_t merged_rows,
                                                              const IndexT *__restrict__ rev, int64_t total,
-                                                             int chunks, uint4 *__restrict__ out, int64_t items) {
-    const int64_t id = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+                                                             int chunks, uint4 *__restrict__ out, int64_t items,
+                                                             FastDiv by_chunks) {
+    const uint32_t id = blockIdx.x * kThreads + threadIdx.x;        // items < 2^31 (checked by the host)
     if (id >= items) return;
-    const int64_t quad = id / chunks;
+    const uint32_t quad = fast_div(id, by_chunks);
     const int chunk = static_cast<int>(id - quad * chunks);
-    const int64_t i0 = quad * kSplitRows;
+    const int64_t i0 = static_cast<int64_t>(quad) * kSplitRows;
     uint4 v[kSplitRows];
 #pragma unroll
     for (int r = 0; r < kSplitRows; ++r) {
@@ -464,6 +492,13 @@ extern "C" int come_token_merge(const void *tokens, int dtype, int64_t rows, int
     a.group_items = rows * g.groups * a.chunks;
     a.group_blocks = ceil_div(a.group_items, kThreads);
     a.single_items = rows * (g.start + g.tail) * a.chunks;
+    COME_REQUIRE(!vec || (a.group_items < (1ll << 31) && a.single_items < (1ll << 31)), COME_ERR_UNSUPPORTED,
+                 "come_token_merge: more than 2^31 16-byte items in one launch");
+    a.by_chunks = make_fastdiv(a.chunks);
+    a.by_groups = make_fastdiv(g.groups > 0 ? g.groups : 1);
+    a.by_mw = make_fastdiv(g.mw > 0 ? g.mw : 1);
+    a.by_per_row = make_fastdiv(g.start + g.tail > 0 ? g.start + g.tail : 1);
+    a.by_side = make_fastdiv(g.W - g.cov_w > 0 ? g.W - g.cov_w : 1);
     const int64_t blocks = a.group_blocks + ceil_div(a.single_items, kThreads);
     COME_REQUIRE(blocks < (1ll << 31), COME_ERR_UNSUPPORTED, "come_token_merge: problem too large for one launch");
     if (blocks == 0) return COME_OK;
@@ -501,14 +536,15 @@ extern "C" int come_token_split(const void *merged, int dtype, int64_t merged_ro
         const int chunks = static_cast<int>(row_bytes / 16);
         const int64_t items = ceil_div(total, kSplitRows) * chunks;
         const int64_t blocks = ceil_div(items, kThreads);
-        COME_REQUIRE(blocks < (1ll << 31), COME_ERR_UNSUPPORTED, "come_token_split: problem too large for one launch");
+        COME_REQUIRE(items < (1ll << 31), COME_ERR_UNSUPPORTED, "come_token_split: problem too large for one launch");
         const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+        const FastDiv by_chunks = make_fastdiv(chunks);
         if (rev_i64)
             hipLaunchKernelGGL(split_vec_kernel<int64_t>, grid, block, 0, s, static_cast<const uint4 *>(merged),
-                               merged_rows, rev_i64, total, chunks, static_cast<uint4 *>(out), items);
+                               merged_rows, rev_i64, total, chunks, static_cast<uint4 *>(out), items, by_chunks);
         else
             hipLaunchKernelGGL(split_vec_kernel<int32_t>, grid, block, 0, s, static_cast<const uint4 *>(merged),
-                               merged_rows, rev_i32, total, chunks, static_cast<uint4 *>(out), items);
+                               merged_rows, rev_i32, total, chunks, static_cast<uint4 *>(out), items, by_chunks);
     } else {
         const int eb = dtype_bytes(dtype);
         const int64_t blocks = ceil_div(total * chans, kThreads);
