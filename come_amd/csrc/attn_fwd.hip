@@ -2,10 +2,10 @@
 // bias, head_dim 64, for gfx950 (wave64, v_mfma_f32_32x32x16 bf16/f16).
 //
 // Work decomposition
-//   One workgroup (4 wavefronts) owns kBlockM = 128 * QT consecutive queries of one
-//   (segment, head); every wavefront owns QT tiles of 32 queries and walks all keys of
-//   the segment in tiles of 64.  K and V tiles are staged once per workgroup in LDS
-//   (double buffered, one barrier per tile); Q stays in registers.
+//   One workgroup (4 wavefronts) owns 256 consecutive queries of one (segment, head);
+//   every wavefront owns two tiles of 32 queries and walks all keys of the segment in
+//   tiles of 64.  K and V tiles are staged once per workgroup in LDS (four stages, one
+//   barrier per tile); Q stays in registers.
 //
 // Orientation
 //   Scores are produced transposed, S^T = K' Q'^T, so that in the MFMA accumulator
@@ -15,15 +15,15 @@
 //   of O^T += V^T P^T without any data movement; V^T fragments come out of the
 //   row-major V tile with the transposing LDS read ds_read_b64_tr_b16.
 //
-// Bias and tail masking without vector ALU work
-//   K' = [K | t_hi t_mid t_lo 0...] (80 columns) and Q' = [Q | 1 1 1 0...] where
-//   t = float(bias) / softmax_scale split exactly into three 16-bit terms, so the
-//   fifth k-step of the score MFMA adds bias / scale to every score (the reference
-//   adds the same quantity, flash_fwd_kernel.h:30-55).  Keys beyond the end of the
-//   segment get t_hi = -inf, which makes their scores -inf and their probabilities 0.
+// Bias, reference point and tail masking without vector ALU work
+//   K' = [K | b_hi b_mid b_lo 1 1 1 0 0] (80 columns) and Q' = [c Q | 1 1 1 -m_hi -m_mid -m_lo 0 0]
+//   with c = softmax_scale log2(e), b = float(bias) log2(e) and m the reference point of the
+//   row, b and m each split exactly into three 16-bit terms: after the fifth k-step of the
+//   score MFMA the accumulator is the exponent of exp2.  (The reference adds bias / scale to
+//   the raw scores, flash_fwd_kernel.h:30-55, and subtracts the scaled running maximum inside
+//   exp2, softmax.h:76-88.)  Keys beyond the end of the segment get b_hi = -inf, which makes
+//   their scores -inf and their probabilities 0.
 #include "come_common.h"
-
-#include <cstdlib>
 
 namespace come {
 namespace {
@@ -37,8 +37,6 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int kHeadDim = 64;
 constexpr int kBlockN = 64;          // keys per tile
-constexpr int kKPitch = 88;          // elements per K' row in LDS (64 + 16 bias/zero + 8 pad): 176 B, odd multiple of 16 B
-constexpr int kVPitch = 96;          // elements per V row in LDS: 192 B = 48 banks, 4 rows tile the 64 banks
 constexpr int kThreads = 256;
 constexpr int kBiasPitch = 24;       // elements per key of the bias / ones block (48 B: conflict-free 16-byte reads)
 
@@ -51,7 +49,7 @@ struct AttnArgs {
     int64_t q_rs, q_hs, k_rs, k_hs, v_rs, v_hs, o_rs, o_hs;
     int64_t total;
     int n_heads, n_mblocks, n_units;
-    float scale, scale_log2, inv_scale;
+    float scale_log2;
 };
 
 template <int DT> struct Elem;
@@ -114,209 +112,6 @@ __device__ inline bool locate_block(const AttnArgs &a, int &mblk, int &head, int
     seq = unit / a.n_heads;
     return unit < a.n_units;
 }
-
-template <int DT, int QT>
-__global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnArgs a) {
-    using E = Elem<DT>;
-    constexpr int kBlockM = 128 * QT;
-    __shared__ __attribute__((aligned(16))) uint16_t lds_k[2][kBlockN * kKPitch];
-    __shared__ __attribute__((aligned(16))) uint16_t lds_v[2][kBlockN * kVPitch];
-
-    int mblk, head, seq;
-    if (!locate_block(a, mblk, head, seq)) return;
-    const int seq_start = a.cu[seq];
-    const int L = a.cu[seq + 1] - seq_start;
-    const int q0 = mblk * kBlockM;
-    if (q0 >= L) return;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int h = lane >> 5;          // which half of the wavefront
-    const int r = lane & 31;          // query column / key row inside a 32x32 tile
-
-    // ---- Q fragments (B operand: n = query r, k = head-dim 16 * ks + 8 * h .. + 7)
-    u32x4 qf[QT][4];
-#pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-        const int row = q0 + (wave * QT + qt) * 32 + r;
-        const uint16_t *qp = a.q + static_cast<int64_t>(seq_start + min(row, L - 1)) * a.q_rs + head * a.q_hs + 8 * h;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) qf[qt][ks] = *reinterpret_cast<const u32x4 *>(qp + 16 * ks);
-    }
-    // fifth k-step of Q': ones against the three bias terms (lower half), zeros elsewhere
-    const u32x4 q_ext = h == 0 ? u32x4{E::kOne | (E::kOne << 16), E::kOne, 0u, 0u} : zero4();
-
-    // ---- staging of one K'/V tile: thread -> (row sr and sr + 32, 16-byte chunk sc)
-    const int sc = tid & 7;
-    const int sr = tid >> 3;
-    const uint16_t *k_base = a.k + static_cast<int64_t>(seq_start) * a.k_rs + head * a.k_hs + sc * 8;
-    const uint16_t *v_base = a.v + static_cast<int64_t>(seq_start) * a.v_rs + head * a.v_hs + sc * 8;
-    const uint16_t *b_base = a.bias ? a.bias + seq_start : nullptr;
-
-    u32x4 k_stage[2], v_stage[2], b_stage;
-    auto fetch = [&](int n0) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int key = n0 + sr + 32 * i;
-            const bool ok = key < L;
-            k_stage[i] = ok ? *reinterpret_cast<const u32x4 *>(k_base + static_cast<int64_t>(key) * a.k_rs) : zero4();
-            v_stage[i] = ok ? *reinterpret_cast<const u32x4 *>(v_base + static_cast<int64_t>(key) * a.v_rs) : zero4();
-        }
-        if (tid < kBlockN) {
-            const int key = n0 + tid;
-            uint32_t t_hi = E::kNegInf, t_mid = 0, t_lo = 0;
-            if (key < L) {
-                const float t = b_base ? E::to_f32(b_base[key]) * a.inv_scale : 0.f;
-                t_hi = E::from_f32(t);
-                const float hi_f = E::to_f32(static_cast<uint16_t>(t_hi));
-                if (fabsf(hi_f) != INFINITY) {                               // an infinite bias stays a single term
-                    const float r1 = t - hi_f;
-                    t_mid = E::from_f32(r1);
-                    t_lo = E::from_f32(r1 - E::to_f32(static_cast<uint16_t>(t_mid)));
-                }
-            }
-            b_stage = u32x4{t_hi | (t_mid << 16), t_lo, 0u, 0u};
-        }
-    };
-    auto commit = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            *reinterpret_cast<u32x4 *>(&lds_k[buf][(sr + 32 * i) * kKPitch + sc * 8]) = k_stage[i];
-            *reinterpret_cast<u32x4 *>(&lds_v[buf][(sr + 32 * i) * kVPitch + sc * 8]) = v_stage[i];
-        }
-        if (tid < kBlockN) {
-            *reinterpret_cast<u32x4 *>(&lds_k[buf][tid * kKPitch + 64]) = b_stage;
-            *reinterpret_cast<u32x4 *>(&lds_k[buf][tid * kKPitch + 72]) = zero4();
-        }
-    };
-
-    // ---- running state per query tile
-    f32x16 o_acc[QT][2];
-    float m_run[QT], l_run[QT];
-#pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-#pragma unroll
-        for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) o_acc[qt][dt][i] = 0.f;
-        m_run[qt] = -INFINITY;
-        l_run[qt] = 0.f;
-    }
-
-    const int n_tiles = (L + kBlockN - 1) / kBlockN;
-    fetch(0);
-    commit(0);
-    __syncthreads();
-
-    // LDS read offsets of this lane
-    const int k_off = r * kKPitch + 8 * h;                                   // + 32*mt*pitch + 16*ks
-    const int v_off = (4 * h + ((lane & 15) >> 2)) * kVPitch + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-
-    for (int j = 0; j < n_tiles; ++j) {
-        const int buf = j & 1;
-        const bool more = j + 1 < n_tiles;
-        if (more) fetch((j + 1) * kBlockN);
-
-        // ---- S^T = K' Q'^T : [64 keys] x [32 * QT queries]
-        f32x16 s_acc[QT][2];
-        const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < 5; ++ks) {
-            const u32x4 kf0 = *reinterpret_cast<const u32x4 *>(&lds_k[buf][k_off + 16 * ks]);
-            const u32x4 kf1 = *reinterpret_cast<const u32x4 *>(&lds_k[buf][k_off + 32 * kKPitch + 16 * ks]);
-#pragma unroll
-            for (int qt = 0; qt < QT; ++qt) {
-                const u32x4 qb = ks < 4 ? qf[qt][ks < 4 ? ks : 0] : q_ext;
-                s_acc[qt][0] = E::mfma(kf0, qb, ks == 0 ? zero16 : s_acc[qt][0]);
-                s_acc[qt][1] = E::mfma(kf1, qb, ks == 0 ? zero16 : s_acc[qt][1]);
-            }
-        }
-
-        // ---- online softmax, in the exp2 domain
-        u32x4 p_frag[QT][4];                                                  // P^T as B operand, one per 16-key step
-#pragma unroll
-        for (int qt = 0; qt < QT; ++qt) {
-            float mx = s_acc[qt][0][0];
-#pragma unroll
-            for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s_acc[qt][0][i]);
-#pragma unroll
-            for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[qt][1][i]);
-            mx = max_across_halves(mx);
-            const float m_new = fmaxf(m_run[qt], mx);
-            const float m_use = m_new == -INFINITY ? 0.f : m_new;            // row fully masked so far
-            const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_use) * a.scale_log2);
-            const float mc = m_use * a.scale_log2;
-            float sum = 0.f;
-#pragma unroll
-            for (int mt = 0; mt < 2; ++mt) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[qt][mt][i], a.scale_log2, -mc));
-                    s_acc[qt][mt][i] = p;
-                    sum += p;
-                }
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    u32x4 f;
-#pragma unroll
-                    for (int w = 0; w < 4; ++w) f[w] = E::pack2(s_acc[qt][mt][8 * t + 2 * w], s_acc[qt][mt][8 * t + 2 * w + 1]);
-                    p_frag[qt][2 * mt + t] = f;
-                }
-            }
-            l_run[qt] = l_run[qt] * alpha + sum;
-            if (__any(m_new != m_run[qt])) {                                  // rescale O only when some row max moved
-#pragma unroll
-                for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) o_acc[qt][dt][i] *= alpha;
-            }
-            m_run[qt] = m_new;
-        }
-
-        // ---- O^T += V^T P^T
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-#pragma unroll
-            for (int dt = 0; dt < 2; ++dt) {
-                const uint16_t *vp = &lds_v[buf][v_off + (16 * u) * kVPitch + 32 * dt];
-                const s16x4 lo = lds_read_tr(vp);
-                const s16x4 hi = lds_read_tr(vp + 8 * kVPitch);
-                const u32x2 lo2 = __builtin_bit_cast(u32x2, lo);
-                const u32x2 hi2 = __builtin_bit_cast(u32x2, hi);
-                const u32x4 vf = u32x4{lo2[0], lo2[1], hi2[0], hi2[1]};
-#pragma unroll
-                for (int qt = 0; qt < QT; ++qt) o_acc[qt][dt] = E::mfma(vf, p_frag[qt][u], o_acc[qt][dt]);
-            }
-        }
-
-        if (more) commit(buf ^ 1);
-        __syncthreads();
-    }
-
-    // ---- epilogue: normalise, write O (and LSE)
-#pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-        const float l_tot = sum_across_halves(l_run[qt]);
-        const float inv = 1.0f / l_tot;
-        const int row = q0 + (wave * QT + qt) * 32 + r;
-        if (row < L) {
-            uint16_t *op = a.out + static_cast<int64_t>(seq_start + row) * a.o_rs + head * a.o_hs + 4 * h;
-#pragma unroll
-            for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    u32x2 w;
-                    w[0] = E::pack2(o_acc[qt][dt][4 * g] * inv, o_acc[qt][dt][4 * g + 1] * inv);
-                    w[1] = E::pack2(o_acc[qt][dt][4 * g + 2] * inv, o_acc[qt][dt][4 * g + 3] * inv);
-                    *reinterpret_cast<u32x2 *>(op + 32 * dt + 8 * g) = w;
-                }
-            if (h == 0 && a.lse)
-                a.lse[static_cast<int64_t>(head) * a.total + seq_start + row] = m_run[qt] * a.scale + __logf(l_tot);
-        }
-    }
-}
-
 
 // -------------------------------------------------------------------------------------
 // Software-pipelined kernel: kBlockM = 256 queries per workgroup, two query tiles per
@@ -595,14 +390,9 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
         };
         auto issue = [&](int m) __attribute__((always_inline)) {
             const int f = m >> 1, qt = m & 1;
-#ifdef COME_EXP_NO_MFMA
-            if (f >= 0) return;
-#endif
             // empty asm statements are ordering pins: MFMAs and exponentials are pure operations which the
             // compiler would otherwise float out of their chunk (sched_barrier only fences what is already there)
-#ifndef COME_EXP_NO_FRAG_PIN
             if (qt == 0) asm volatile("" : "+v"(frag[f]));
-#endif
             if (f < 4) {
                 const int u = f >> 1, dt = f & 1;
                 o_acc[qt][dt] = E::mfma(frag[f], p_frag[Y][qt][u], o_acc[qt][dt]);
@@ -638,19 +428,9 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
                 sum[qt] = E::dot2_ones(pw, sum[qt]);
             }
             float s0 = s_acc[X][c >> 3][2 * (c & 7)], s1 = s_acc[X][c >> 3][2 * (c & 7) + 1];
-#ifdef COME_EXP_S_PIN
-            asm volatile("" : "+v"(s0), "+v"(s1));
-#endif
-#ifdef COME_EXP_NO_EXP
-            p0 = s0;
-            p1 = s1;
-#else
             p0 = __builtin_amdgcn_exp2f(s0);
             p1 = __builtin_amdgcn_exp2f(s1);
-#endif
-#ifndef COME_EXP_NO_P_PIN
             asm volatile("" : "+v"(p0), "+v"(p1));
-#endif
             __builtin_amdgcn_sched_barrier(0);
         }
         {
@@ -765,46 +545,21 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
 
     for (int j = 0; j < n_tiles; ++j) {
         const int kb = j & 3, kb1 = (j + 1) & 3, kb2 = (j + 2) & 3, kb3 = (j + 3) & 3;   // stage of tile j, j+1, ..
-#ifndef COME_EXP_NO_STAGE
         load_bias(j + 4, kb);          // raw bias runs one more tile ahead (converted between the slots of iteration j+2)
         stage_k(j + 3, kb3);           // K'(j+3) replaces K'(j-1), V(j+2) replaces V(j-2): both idle since the
         stage_v(j + 2, kb2);           // last barrier; they are first read two barriers from now
-#endif
         float sum[2];
         peek_bias(kb2);
-#ifdef COME_EXP_TIMING
-        const uint64_t t_a = __builtin_readcyclecounter();
-#endif
         // slot a: keys 0..31 of tile j become probabilities; scores of keys 32..63; P V of keys 32..63 of tile j-1
         slot(0, 1, kb, 1, kb3, 1, sum);
         finish_slot(1, sum);
-#ifndef COME_EXP_NO_STAGE
         commit_bias(j + 2, kb2);       // raw bias landed before the last barrier; published by the next one
-#endif
         // slot b: keys 32..63 of tile j become probabilities; scores of keys 0..31 of tile j+1; P V of keys 0..31 of tile j
-#ifdef COME_EXP_TIMING
-        const uint64_t t_b = __builtin_readcyclecounter();
-#endif
         slot(1, 0, kb1, 0, kb, 0, sum);
         finish_slot(0, sum);
-#ifdef COME_EXP_TIMING
-        const uint64_t t_c = __builtin_readcyclecounter();
-#endif
 
         staged_wait(true);             // loads issued one iteration ago have landed
-#ifndef COME_EXP_NO_BARRIER
         __syncthreads();
-#endif
-#ifdef COME_EXP_TIMING
-        if (a.lse && blockIdx.x == 1000 && lane == 0 && j >= 100 && j < 132) {
-            const uint64_t t_d = __builtin_readcyclecounter();
-            float *dump = a.lse + (wave * 32 + (j - 100)) * 4;
-            dump[0] = static_cast<float>(t_b - t_a);
-            dump[1] = static_cast<float>(t_c - t_b);
-            dump[2] = static_cast<float>(t_d - t_c);
-            dump[3] = static_cast<float>(t_d & 0xffffff);
-        }
-#endif
     }
     pv_mfma(1, (n_tiles - 1) & 3, 1);      // keys 32..63 of the last tile
 #pragma unroll
@@ -877,9 +632,7 @@ extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v,
                      (reinterpret_cast<uintptr_t>(v) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0,
                  COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: q/k/v must be 16-byte aligned, out 8-byte aligned");
 
-    static const int QT = getenv("COME_ATTN_QT") ? atoi(getenv("COME_ATTN_QT")) : 2;
-    static const bool kPipe = getenv("COME_ATTN_PIPE") ? atoi(getenv("COME_ATTN_PIPE")) != 0 : true;
-    const int kBlockM = kPipe ? 256 : 128 * QT;
+    constexpr int kBlockM = 256;
     AttnArgs a{};
     a.q = static_cast<const uint16_t *>(q);
     a.k = static_cast<const uint16_t *>(k);
@@ -895,23 +648,14 @@ extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v,
     a.total = total;
     a.n_heads = static_cast<int>(n_heads);
     a.n_mblocks = static_cast<int>(ceil_div(max_seqlen, kBlockM));
-    a.scale = softmax_scale;
     a.scale_log2 = softmax_scale * 1.4426950408889634f;
-    a.inv_scale = 1.0f / softmax_scale;
     a.n_units = static_cast<int>(n_seq * n_heads);
     const int64_t n_wg = ceil_div(n_seq * n_heads, 8) * 8 * a.n_mblocks;
     COME_REQUIRE(n_wg < (1ll << 31), COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: grid too large");
     const dim3 grid(static_cast<unsigned>(n_wg)), block(kThreads);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (kPipe) {
-        if (dtype == COME_BF16) hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_BF16>), grid, block, 0, s, a);
-        else hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_F16>), grid, block, 0, s, a);
-    } else if (dtype == COME_BF16) {
-        if (QT == 1) hipLaunchKernelGGL((attn_fwd_kernel<COME_BF16, 1>), grid, block, 0, s, a);
-        else hipLaunchKernelGGL((attn_fwd_kernel<COME_BF16, 2>), grid, block, 0, s, a);
-    } else {
-        hipLaunchKernelGGL((attn_fwd_kernel<COME_F16, 2>), grid, block, 0, s, a);
-    }
+    if (dtype == COME_BF16) hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_BF16>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_F16>), grid, block, 0, s, a);
     COME_CHECK_LAUNCH("come_attn_varlen_fwd");
     return COME_OK;
 }
