@@ -41,6 +41,9 @@ SIGNATURES = {
                                     _ptr, _i64, _i64, _ptr, _ptr]),
     "come_qk_norm_rope": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                  _int, _ptr, _ptr, _ptr, _ptr, _f32, _ptr, _ptr, _ptr, _i64, _ptr]),
+    "come_jagged_add_suffix": (_int, [_ptr, _ptr, _int, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr]),
+    "come_jagged_split_suffix": (_int, [_ptr, _ptr, _int, _i64, _i64, _ptr, _i64, _i64, _ptr, _ptr, _ptr, _ptr,
+                                        _ptr]),
 }
 
 _lock = threading.Lock()

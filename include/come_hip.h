@@ -206,6 +206,29 @@ int come_qk_norm_rope(void *q, void *k, int dtype,
                       const int64_t *positions, const void *cos_table, const void *sin_table,
                       int64_t n_pos, void *stream);
 
+/*
+ * come_jagged_add_suffix / come_jagged_split_suffix — append `count` dense rows to every packed
+ * segment, or strip the last `count` rows of every segment again.
+ *
+ *   tokens   [rows, chans] of `dtype`, weight [rows] float (may be NULL together with out_weight)
+ *   offsets  [n_seg + 1] int64 segment boundaries of the input, offsets[n_seg] == rows
+ *   add:     suffix [n_seg, count, chans]; out_tokens [rows + n_seg * count, chans]: segment m
+ *            followed by suffix[m]; appended rows get weight 1; out_offsets[m] = offsets[m] + m * count
+ *   split:   out_tokens [rows - n_seg * count, chans], out_suffix [n_seg, count, chans] = the last
+ *            `count` rows of each segment, out_offsets[m] = offsets[m] - m * count.  Every segment
+ *            must hold at least `count` rows (the caller checks: it needs the offsets on the host).
+ *
+ * Stand in for JaggedTokens.add_suffix / split_suffix (src/interface/token_merger.py:23-58, 60-100),
+ * which the reference runs as arange / searchsorted / index_copy_ / index_select tensor passes.
+ */
+int come_jagged_add_suffix(const void *tokens, const float *weight, int dtype, int64_t rows, int64_t chans,
+                           const int64_t *offsets, int64_t n_seg, const void *suffix, int64_t count,
+                           void *out_tokens, float *out_weight, int64_t *out_offsets, void *stream);
+int come_jagged_split_suffix(const void *tokens, const float *weight, int dtype, int64_t rows, int64_t chans,
+                             const int64_t *offsets, int64_t n_seg, int64_t count,
+                             void *out_tokens, float *out_weight, int64_t *out_offsets, void *out_suffix,
+                             void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -33,6 +33,8 @@ Pinning status of each function (what fixes its answers besides this text):
                                       the reference's tests; reductions to
                                       torch SDPA, key-duplication identity,
                                       logsumexp identity.
+  add_suffix / split_suffix           the reference's 3 known-answer cases
+                                      (tests/golden/suffix.json), round trip.
   qk_norm_rope / rope_2d              layer_norm is the library routine; the
                                       rotation is PARITY UNPINNED by the
                                       reference's tests and pinned here by
@@ -41,7 +43,7 @@ Pinning status of each function (what fixes its answers besides this text):
                                       property of q.k).
 """
 
-from .jagged import JaggedTokens  # noqa: F401
+from .jagged import JaggedTokens, add_suffix, split_suffix  # noqa: F401
 from .token_merge import (  # noqa: F401
     token_merge_1d,
     token_merge_2d,

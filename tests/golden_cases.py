@@ -27,3 +27,18 @@ def _tensorize(case):
 
 MERGE_1D = [_tensorize(c) for c in _load("merge_1d.json")]
 MERGE_2D = [_tensorize(c) for c in _load("merge_2d.json")]
+
+
+def _tensorize_suffix(case):
+    out = dict(case)
+    out["tokens"] = torch.tensor(case["tokens"], dtype=torch.float32).unsqueeze(0)
+    out["weight"] = torch.tensor(case["weight"], dtype=torch.float32)
+    out["offset"] = torch.tensor(case["offset"], dtype=torch.int64)
+    out["suffix"] = torch.tensor(case["suffix"], dtype=torch.float32)
+    out["out"] = torch.tensor(case["out"], dtype=torch.float32).unsqueeze(0)
+    out["out_weight"] = torch.tensor(case["out_weight"], dtype=torch.float32)
+    out["out_offset"] = torch.tensor(case["out_offset"], dtype=torch.int64)
+    return out
+
+
+SUFFIX = [_tensorize_suffix(c) for c in _load("suffix.json")]
