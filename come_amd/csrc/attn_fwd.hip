@@ -37,7 +37,6 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int kHeadDim = 64;
 constexpr int kBlockN = 64;          // keys per tile
-constexpr int kThreads = 256;
 constexpr int kBiasPitch = 24;       // elements per key of the bias / ones block (48 B: conflict-free 16-byte reads)
 
 struct AttnArgs {
@@ -153,10 +152,13 @@ __device__ inline uint32_t lds_address(const void *p) {
 }
 constexpr float kSumLimit = 16777216.f;      // 2^24: a tile row sum above this moves the reference point
 
-template <int DT>
-__global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs a) {
+template <int DT, int NW>
+__global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a) {
     using E = Elem<DT>;
-    constexpr int kBlockM = 256;
+    static_assert(NW == 4 || NW == 8, "4 or 8 wavefronts per workgroup");
+    constexpr int kBlockM = 64 * NW;           // queries per workgroup
+    constexpr int kThreads = 64 * NW;
+    constexpr int kDma = 8 / NW;               // direct loads per wavefront for one K (or V) tile
     // K and V tiles: 64 rows of 128 bytes, unpadded, filled by direct global->LDS loads (a wavefront's
     // load lands as 1 KiB in lane order); bank conflicts are avoided by permuting the 16-byte chunks
     // inside a row: K chunk c of row r sits at slot c ^ ((r >> 1) & 7), V chunk c at c ^ (((r >> 1) & 1) << 2).
@@ -212,11 +214,11 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
     const char *b_seg = a.bias ? reinterpret_cast<const char *>(b_addr & ~static_cast<uintptr_t>(3)) : nullptr;
     const uint32_t b_mis = static_cast<uint32_t>(b_addr & 3);
     const uint32_t k_rs_b = static_cast<uint32_t>(a.k_rs) * 2u, v_rs_b = static_cast<uint32_t>(a.v_rs) * 2u;
-    uint32_t k_goff[2], v_goff[2], k_chunk[2], v_chunk[2];
-    int st_row[2];
+    uint32_t k_goff[kDma], v_goff[kDma], k_chunk[kDma], v_chunk[kDma];
+    int st_row[kDma];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        st_row[i] = 8 * (2 * wave + i) + (lane >> 3);
+    for (int i = 0; i < kDma; ++i) {
+        st_row[i] = 8 * (kDma * wave + i) + (lane >> 3);
         k_chunk[i] = static_cast<uint32_t>((lane & 7) ^ ((st_row[i] >> 1) & 7)) * 16u;
         v_chunk[i] = static_cast<uint32_t>((lane & 7) ^ (((st_row[i] >> 1) & 1) << 2)) * 16u;
         k_goff[i] = static_cast<uint32_t>(st_row[i]) * k_rs_b + k_chunk[i];
@@ -230,10 +232,10 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
         const uint32_t tile_off = static_cast<uint32_t>(tile) * k_tile_step;         // wave-uniform
         const bool full = n0 + kBlockN <= L;                                        // wave-uniform
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < kDma; ++i) {
             uint32_t off = tile_off + k_goff[i];
             if (!full) off = n0 + st_row[i] < L ? off : k_last + k_chunk[i];
-            dma_b128(k_seg, off, lds_address(&lds_k[buf][(2 * wave_u + i) * 512]));
+            dma_b128(k_seg, off, lds_address(&lds_k[buf][(kDma * wave_u + i) * 512]));
         }
     };
     // raw bias of the 64 keys of a tile: wavefront 0 brings the aligned 32-bit word that holds each key's
@@ -249,10 +251,10 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
         const uint32_t tile_off = static_cast<uint32_t>(tile) * v_tile_step;
         const bool full = n0 + kBlockN <= L;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < kDma; ++i) {
             uint32_t off = tile_off + v_goff[i];
             if (!full) off = n0 + st_row[i] < L ? off : v_last + v_chunk[i];
-            dma_b128(v_seg, off, lds_address(&lds_v[buf][(2 * wave_u + i) * 512]));
+            dma_b128(v_seg, off, lds_address(&lds_v[buf][(kDma * wave_u + i) * 512]));
         }
     };
     // exact three-term 16-bit split of an fp32 value (an infinite value stays one term)
@@ -295,10 +297,13 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_pipe_kernel(const AttnArgs 
         }
     };
     auto staged_wait = [&](bool with_bias_load) __attribute__((always_inline)) {
+        // the direct loads issued in this iteration (K, V and, on wavefront 0, the bias) may stay in flight
         if (with_bias_load && wave_u == 0 && b_seg) {
-            asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+            if (NW == 4) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
         } else {
-            asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+            if (NW == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
         }
     };
 
@@ -632,7 +637,24 @@ extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v,
                      (reinterpret_cast<uintptr_t>(v) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0,
                  COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: q/k/v must be 16-byte aligned, out 8-byte aligned");
 
-    constexpr int kBlockM = 256;
+    // 8 wavefronts per workgroup share every staged K / V tile among 512 queries (half the L2 -> LDS traffic),
+    // but such a workgroup fills a whole CU, so a partly filled last round of workgroups costs a full round.
+    // It is used for long segments when the expected number of workgroups nearly fills its last round;
+    // otherwise two 256-query workgroups share a CU and the last round finishes early on the CUs it uses.
+    bool wide = false;
+    if (max_seqlen >= 4096) {
+        static const int n_cu = [] {
+            int dev = 0, n = 0;
+            if (hipGetDevice(&dev) != hipSuccess ||
+                hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+                n = 256;
+            return n;
+        }();
+        const int64_t expected = n_heads * ceil_div(total + n_seq * 256, 512);
+        const int64_t rounds = ceil_div(expected, n_cu);
+        wide = expected * 100 >= rounds * n_cu * 95;
+    }
+    const int kBlockM = wide ? 512 : 256;
     AttnArgs a{};
     a.q = static_cast<const uint16_t *>(q);
     a.k = static_cast<const uint16_t *>(k);
@@ -652,10 +674,15 @@ extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v,
     a.n_units = static_cast<int>(n_seq * n_heads);
     const int64_t n_wg = ceil_div(n_seq * n_heads, 8) * 8 * a.n_mblocks;
     COME_REQUIRE(n_wg < (1ll << 31), COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: grid too large");
-    const dim3 grid(static_cast<unsigned>(n_wg)), block(kThreads);
+    const dim3 grid(static_cast<unsigned>(n_wg)), block(wide ? 512 : 256);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == COME_BF16) hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_BF16>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_F16>), grid, block, 0, s, a);
+    if (wide) {
+        if (dtype == COME_BF16) hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_BF16, 8>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_F16, 8>), grid, block, 0, s, a);
+    } else {
+        if (dtype == COME_BF16) hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_BF16, 4>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_F16, 4>), grid, block, 0, s, a);
+    }
     COME_CHECK_LAUNCH("come_attn_varlen_fwd");
     return COME_OK;
 }
