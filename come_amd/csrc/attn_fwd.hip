@@ -8,21 +8,21 @@
 //   barrier per tile); Q stays in registers.
 //
 // Orientation
-//   Scores are produced transposed, S^T = K' Q'^T, so that in the MFMA accumulator
+//   Scores are produced transposed, S^T = K (c Q)^T, so that in the MFMA accumulator
 //   layout a lane holds ONE query (lane % 32) and 16 keys per 32x32 tile: the row max
 //   and row sum of the online softmax are in-lane reductions plus one exchange between
 //   lane l and lane l ^ 32.  The same registers, rounded to 16 bit, are the B operand
 //   of O^T += V^T P^T without any data movement; V^T fragments come out of the
 //   row-major V tile with the transposing LDS read ds_read_b64_tr_b16.
 //
-// Bias, reference point and tail masking without vector ALU work
-//   K' = [K | b_hi b_mid b_lo 1 1 1 0 0] (80 columns) and Q' = [c Q | 1 1 1 -m_hi -m_mid -m_lo 0 0]
-//   with c = softmax_scale log2(e), b = float(bias) log2(e) and m the reference point of the
-//   row, b and m each split exactly into three 16-bit terms: after the fifth k-step of the
-//   score MFMA the accumulator is the exponent of exp2.  (The reference adds bias / scale to
-//   the raw scores, flash_fwd_kernel.h:30-55, and subtracts the scaled running maximum inside
-//   exp2, softmax.h:76-88.)  Keys beyond the end of the segment get b_hi = -inf, which makes
-//   their scores -inf and their probabilities 0.
+// Bias, reference point and tail masking
+//   The accumulator of a score tile does not start from zero but from b_k - m_q, with
+//   b = float(bias) log2(e) of the key (read from LDS, -inf beyond the end of the segment) and
+//   m the reference point of the query's row, and Q is multiplied by c = softmax_scale log2(e)
+//   once: after the four k-steps of the score MFMA the accumulator is the exponent of exp2.
+//   (The reference adds bias / scale to the raw scores, flash_fwd_kernel.h:30-55, and
+//   subtracts the scaled running maximum inside exp2, softmax.h:76-88.)  Keys beyond the end of
+//   the segment get scores of -inf and probabilities of exactly 0.
 #include "come_common.h"
 
 namespace come {
@@ -30,6 +30,7 @@ namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -37,7 +38,6 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int kHeadDim = 64;
 constexpr int kBlockN = 64;          // keys per tile
-constexpr int kBiasPitch = 24;       // elements per key of the bias / ones block (48 B: conflict-free 16-byte reads)
 
 struct AttnArgs {
     const uint16_t *q, *k, *v;
@@ -53,7 +53,7 @@ struct AttnArgs {
 
 template <int DT> struct Elem;
 template <> struct Elem<COME_BF16> {
-    static constexpr uint32_t kOne = 0x3F80u, kNegInf = 0xFF80u;
+    static constexpr uint32_t kOne = 0x3F80u;
     __device__ static inline float to_f32(uint16_t x) { return __uint_as_float(static_cast<uint32_t>(x) << 16); }
     __device__ static inline uint16_t from_f32(float x) { return static_cast<uint16_t>(pack2_bf16(x, 0.f) & 0xffffu); }
     __device__ static inline uint32_t pack2(float lo, float hi) { return pack2_bf16(lo, hi); }
@@ -67,7 +67,7 @@ template <> struct Elem<COME_BF16> {
     }
 };
 template <> struct Elem<COME_F16> {
-    static constexpr uint32_t kOne = 0x3C00u, kNegInf = 0xFC00u;
+    static constexpr uint32_t kOne = 0x3C00u;
     __device__ static inline float to_f32(uint16_t x) { return __half2float(__builtin_bit_cast(__half, x)); }
     __device__ static inline uint16_t from_f32(float x) { return __builtin_bit_cast(uint16_t, __float2half_rn(x)); }
     __device__ static inline uint32_t pack2(float lo, float hi) { return pack2_f16(lo, hi); }
@@ -118,21 +118,20 @@ __device__ inline bool locate_block(const AttnArgs &a, int &mblk, int &head, int
 // into probabilities, the matrix pipe runs the score MFMAs (next key tile) and the P V MFMAs
 // (current key tile) of the other one:
 //
-//   slot a(j): VALU P0 = exp2(S0(j))      MFMA S1(j) = K'(j) Q1'^T ; O1 += V(j-1)^T P1(j-1)
-//   slot b(j): VALU P1 = exp2(S1(j))      MFMA S0(j+1) = K'(j+1) Q0'^T ; O0 += V(j)^T P0(j)
+//   slot a(j): VALU P0 = exp2(S0(j))      MFMA S1(j) = K(j) Q1^T ; O1 += V(j-1)^T P1(j-1)
+//   slot b(j): VALU P1 = exp2(S1(j))      MFMA S0(j+1) = K(j+1) Q0^T ; O0 += V(j)^T P0(j)
 //
-// K' tiles j, j+1 and V tiles j-1, j are live in one iteration and the tiles of the next iteration
+// K tiles j, j+1 and V tiles j-1, j are live in one iteration and the tiles of the next iteration
 // are in flight from global memory, so LDS holds four tiles of each; one barrier per iteration.
 //
 // Scores leave the MFMA already in the form the exponential needs:
 //   S'' = (c q) . k + bias log2(e) - m,      c = softmax_scale log2(e)
-// Q is multiplied by c once (and rounded back to 16 bit); bias log2(e) and the reference point m of
-// the row ride through the fifth k-step as exact three-term 16-bit splits (K' carries the bias terms
-// and ones, Q' carries ones and the terms of -m).  m is the row maximum of the first key tile and is
-// moved, by a power of two, only when a half-tile's row sum leaves a safe range (sums and outputs are
-// then rescaled as in the usual online softmax); softmax is invariant to the choice of m, and fp32 / 16-bit floats
-// keep full relative precision for probabilities above 1.  The steady state therefore spends one
-// exp2, half a pack and half a dot per score on the vector ALU and nothing else.
+// Q is multiplied by c once (and rounded back to 16 bit); bias log2(e) - m is the initial value of the
+// accumulator (one subtraction per score on the vector ALU).  m is the row maximum of the first 32 keys and
+// is moved, by a power of two, only when a half-tile's row sum leaves a safe range (sums and outputs are
+// then rescaled as in the usual online softmax); softmax is invariant to the choice of m, and fp32 / 16-bit
+// floats keep full relative precision for probabilities above 1.  The steady state therefore spends one
+// subtraction, one exp2, half a pack and half a dot per score on the vector ALU and nothing else.
 // -------------------------------------------------------------------------------------
 constexpr int kStages = 4;
 
@@ -162,11 +161,12 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     // K and V tiles: 64 rows of 128 bytes, unpadded, filled by direct global->LDS loads (a wavefront's
     // load lands as 1 KiB in lane order); bank conflicts are avoided by permuting the 16-byte chunks
     // inside a row: K chunk c of row r sits at slot c ^ ((r >> 1) & 7), V chunk c at c ^ (((r >> 1) & 1) << 2).
-    // lds_b: per key 48 bytes, [bias terms and ones (16 B) | zeros (16 B) | pad], the fifth k-step of K'.
+    // lds_b: per key one float, bias log2(e) (-inf beyond the end of the segment): the initial value of its scores.
     __shared__ __attribute__((aligned(1024))) uint16_t lds_k[kStages][kBlockN * kHeadDim];
     __shared__ __attribute__((aligned(1024))) uint16_t lds_v[kStages][kBlockN * kHeadDim];
-    __shared__ __attribute__((aligned(16))) uint16_t lds_b[kStages][kBlockN * kBiasPitch];
+    __shared__ __attribute__((aligned(16))) float lds_b[kStages][kBlockN];
     __shared__ __attribute__((aligned(256))) uint32_t lds_braw[kStages][kBlockN];   // raw bias words as loaded
+    __shared__ float lds_ref[NW];                                                   // prologue: reference point per wavefront
 
     int mblk, head, seq;
     if (!locate_block(a, mblk, head, seq)) return;
@@ -197,11 +197,6 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
                                          E::to_f32(static_cast<uint16_t>(raw[w] >> 16)) * a.scale_log2);
         }
     }
-    // fifth k-step of Q' (lower half-wave only): [1 1 1 | -m split in three | 0 0]
-    u32x4 q_ext[2];
-    q_ext[0] = h == 0 ? u32x4{E::kOne | (E::kOne << 16), E::kOne, 0u, 0u} : zero4();
-    q_ext[1] = q_ext[0];
-
     // ---- global -> LDS staging.  Wavefront w fills rows 16 w .. 16 w + 15 of a tile with two direct
     // loads; lane l of load i brings row 8 (2 w + i) + l / 8, slot l % 8.  A key index beyond the segment
     // is redirected to its last key (finite data); such keys get a bias term of -inf, so their
@@ -239,7 +234,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
         }
     };
     // raw bias of the 64 keys of a tile: wavefront 0 brings the aligned 32-bit word that holds each key's
-    // 16-bit bias; it is converted into the fifth k-step block two iterations later (commit_bias)
+    // 16-bit bias; it is converted to a float two iterations later (commit_bias)
     auto load_bias = [&](int tile, int buf) __attribute__((always_inline)) {
         if (wave_u == 0 && b_seg) {
             const uint32_t key = static_cast<uint32_t>(min(tile * kBlockN + lane, L - 1));
@@ -257,21 +252,9 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
             dma_b128(v_seg, off, lds_address(&lds_v[buf][(kDma * wave_u + i) * 512]));
         }
     };
-    // exact three-term 16-bit split of an fp32 value (an infinite value stays one term)
-    auto split3 = [&](float t, uint32_t &t_hi, uint32_t &t_mid, uint32_t &t_lo) __attribute__((always_inline)) {
-        t_hi = E::from_f32(t);
-        t_mid = 0;
-        t_lo = 0;
-        const float hi_f = E::to_f32(static_cast<uint16_t>(t_hi));
-        if (fabsf(hi_f) != INFINITY) {
-            const float r1 = t - hi_f;
-            t_mid = E::from_f32(r1);
-            t_lo = E::from_f32(r1 - E::to_f32(static_cast<uint16_t>(t_mid)));
-        }
-    };
     // conversion of the raw bias of one tile, split in two so that the LDS read is in flight during a slot:
-    // peek_bias() requests the word, commit_bias() converts it and writes the fifth k-step block
-    // [bias log2(e) in three terms | 1 1 1 | 0 0] followed by 16 bytes of zeros; -inf beyond the segment
+    // peek_bias() requests the word, commit_bias() writes bias log2(e) - m_base as a float, -inf beyond the segment
+    float m_base = 0.f;           // reference point shared by the rows of the workgroup (uniform)
     uint32_t b_word = 0;
     auto peek_bias = [&](int buf) __attribute__((always_inline)) {
         if (wave_u == 0 && b_seg) b_word = lds_braw[buf][lane];
@@ -284,16 +267,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
                 const uint32_t at = b_mis + 2u * static_cast<uint32_t>(min(key, L - 1));
                 bias = E::to_f32(static_cast<uint16_t>((at & 2u) ? (b_word >> 16) : (b_word & 0xffffu)));
             }
-            uint32_t t_hi, t_mid, t_lo;
-            split3(bias * kLog2e, t_hi, t_mid, t_lo);
-            if (key >= L) {
-                t_hi = E::kNegInf;
-                t_mid = 0;
-                t_lo = 0;
-            }
-            *reinterpret_cast<u32x4 *>(&lds_b[buf][lane * kBiasPitch]) =
-                u32x4{t_hi | (t_mid << 16), t_lo | (E::kOne << 16), E::kOne | (E::kOne << 16), 0u};
-            *reinterpret_cast<u32x4 *>(&lds_b[buf][lane * kBiasPitch + 8]) = zero4();
+            lds_b[buf][lane] = key < L ? bias * kLog2e - m_base : -INFINITY;
         }
     };
     auto staged_wait = [&](bool with_bias_load) __attribute__((always_inline)) {
@@ -311,7 +285,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     int k_rd[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) k_rd[ks] = r * kHeadDim + (((2 * ks + h) ^ ((r >> 1) & 7)) << 3);
-    const int b_rd = r * kBiasPitch + 8 * h;
+    const int b_rd = 4 * h;                // keys 8 g + 4 h .. + 3 of a half-tile are accumulator elements 4 g .. 4 g + 3
     const int i16 = lane & 15;
     int v_rd[2];
 #pragma unroll
@@ -326,7 +300,9 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     f32x16 s_acc[2][2];
     f32x16 o_acc[2][2];          // [query tile][head-dim half]
     u32x4 p_frag[2][2][2];
-    float m_run[2] = {0.f, 0.f};  // reference point of the row, log2 units
+    float m_run[2] = {0.f, 0.f};  // reference point of the row, log2 units: m_base + delta
+    float delta[2] = {0.f, 0.f};  // what the row's reference point differs from m_base by (0 for nearly all rows)
+    bool has_delta = false;       // wave-uniform: some row of this wavefront has delta != 0
     float l_run[2] = {0.f, 0.f};  // per-lane partial row sum
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
@@ -339,16 +315,21 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
         }
     }
 
-    // scores of both query tiles against half-tile `half` of the K' tile in `buf`, into buffer b
+    // scores of both query tiles against half-tile `half` of the K tile in `buf`, into buffer b: the accumulators
+    // start from the LDS bias values of their keys and collect the four k-steps of (c Q) K^T
     auto score_mfma = [&](int b, int buf, int half) __attribute__((always_inline)) {
+        f32x16 seed;
 #pragma unroll
-        for (int ks = 0; ks < 5; ++ks) {
-            const uint16_t *kp = ks < 4 ? &lds_k[buf][k_rd[ks < 4 ? ks : 0] + 32 * half * kHeadDim]
-                                        : &lds_b[buf][b_rd + 32 * half * kBiasPitch];
-            const u32x4 kf = *reinterpret_cast<const u32x4 *>(kp);
+        for (int g = 0; g < 4; ++g) {
+            const f32x4 bq = *reinterpret_cast<const f32x4 *>(&lds_b[buf][32 * half + 8 * g + b_rd]);
 #pragma unroll
-            for (int qt = 0; qt < 2; ++qt)
-                s_acc[b][qt] = E::mfma(kf, ks < 4 ? qf[qt][ks < 4 ? ks : 0] : q_ext[qt], ks == 0 ? zero16 : s_acc[b][qt]);
+            for (int e = 0; e < 4; ++e) seed[4 * g + e] = bq[e];
+        }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const u32x4 kf = *reinterpret_cast<const u32x4 *>(&lds_k[buf][k_rd[ks] + 32 * half * kHeadDim]);
+#pragma unroll
+            for (int qt = 0; qt < 2; ++qt) s_acc[b][qt] = E::mfma(kf, qf[qt][ks], ks == 0 ? seed : s_acc[b][qt]);
         }
     };
     // O^T += V^T P^T of both query tiles for half-tile `half` of the V tile in `buf`, probabilities of buffer b
@@ -369,17 +350,18 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
 
     // One slot in explicit issue order.  The vector ALU turns the scores in buffer X (one 32-key half-tile,
     // both query tiles) into probabilities.  Meanwhile the matrix pipe builds the scores of the next
-    // half-tile in buffer Y (10 MFMAs on 5 K' fragments, each fragment shared by both query tiles) and
+    // half-tile in buffer Y (8 MFMAs on 4 K fragments, each fragment shared by both query tiles) and
     // adds the previous half-tile's P V (8 MFMAs on 4 V fragments, probabilities of buffer Y from the
     // previous slot).  Every MFMA is followed by a chunk of vector work and fragments are requested two
     // fragments (four MFMAs) ahead, so an in-order wavefront always has independent work behind each
     // MFMA.  sched_barrier keeps the compiler from regrouping the chunks.
     // Returns through sum[qt] the row sums of this lane over the half-tile.
     auto slot = [&](int X, int Y, int kbuf, int khalf, int vbuf, int vhalf, float (&sum)[2]) __attribute__((always_inline)) {
-        // fragments 0..3: V (u, dt) of the P V MFMAs 0..7; fragments 4..8: K' k-steps of the score MFMAs 8..17.
+        // fragments 0..3: V (u, dt) of the P V MFMAs 0..7; fragments 4..7: K k-steps of the score MFMAs 8..15.
         // P V goes first: the probabilities of buffer Y die while those of buffer X are born, and the score
         // registers of buffer Y are not needed before half of buffer X has been consumed.
-        u32x4 frag[9];
+        u32x4 frag[8];
+        f32x16 seed;                  // bias log2(e) - m_base of this lane's 16 keys of the half-tile being scored
         auto request = [&](int f) __attribute__((always_inline)) {
             if (f < 4) {
                 const int u = f >> 1, dt = f & 1;
@@ -387,10 +369,8 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
                 const u32x2 lo2 = __builtin_bit_cast(u32x2, lds_read_tr(vp));
                 const u32x2 hi2 = __builtin_bit_cast(u32x2, lds_read_tr(vp + 8 * kHeadDim));
                 frag[f] = u32x4{lo2[0], lo2[1], hi2[0], hi2[1]};
-            } else if (f < 9) {
-                const int ks = f - 4;
-                frag[f] = ks < 4 ? *reinterpret_cast<const u32x4 *>(&lds_k[kbuf][k_rd[ks < 4 ? ks : 0] + 32 * khalf * kHeadDim])
-                                 : *reinterpret_cast<const u32x4 *>(&lds_b[kbuf][b_rd + 32 * khalf * kBiasPitch]);
+            } else if (f < 8) {
+                frag[f] = *reinterpret_cast<const u32x4 *>(&lds_k[kbuf][k_rd[f - 4] + 32 * khalf * kHeadDim]);
             }
         };
         auto issue = [&](int m) __attribute__((always_inline)) {
@@ -402,8 +382,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
                 const int u = f >> 1, dt = f & 1;
                 o_acc[qt][dt] = E::mfma(frag[f], p_frag[Y][qt][u], o_acc[qt][dt]);
             } else {
-                const int ks = f - 4;
-                s_acc[Y][qt] = E::mfma(frag[f], ks < 4 ? qf[qt][ks < 4 ? ks : 0] : q_ext[qt], ks == 0 ? zero16 : s_acc[Y][qt]);
+                s_acc[Y][qt] = E::mfma(frag[f], qf[qt][f - 4], f == 4 ? seed : s_acc[Y][qt]);
             }
         };
         request(0);
@@ -413,18 +392,13 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
         float p0 = 0.f, p1 = 0.f;
 #pragma unroll
         for (int c = 0; c < 16; ++c) {
-            // MFMAs 0,1 | 2,3 | 4 | 5 | ... | 17: the last score MFMA is one chunk away from the end of the slot
-            if (c == 0) {
-                issue(0);
-                issue(1);
-                request(2);
-            } else if (c == 1) {
-                issue(2);
-                issue(3);
-                request(3);
-            } else {
-                issue(c + 2);
-                if ((c & 1) == 0) request((c >> 1) + 3);     // chunk 2 -> fragment 4, ..., chunk 10 -> fragment 8
+            // one MFMA per chunk: P V MFMAs 0..7, score MFMAs 8..15; fragments are requested four chunks ahead
+            issue(c);
+            if ((c & 1) == 0 && c <= 10) request((c >> 1) + 2);      // chunk 0 -> fragment 2, ..., chunk 10 -> fragment 7
+            if (c >= 1 && c <= 4) {                                  // initial values of the scores, needed by chunk 8
+                const f32x4 bq = *reinterpret_cast<const f32x4 *>(&lds_b[kbuf][32 * khalf + 8 * (c - 1) + b_rd]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) seed[4 * (c - 1) + e] = bq[e];
             }
             if (c > 0) {                    // pack and add the pair whose exponentials were issued one chunk ago
                 const int pc = c - 1, qt = pc >> 3, w = pc & 7;
@@ -448,15 +422,6 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
         asm volatile("" : "+v"(sum[1]) : "v"(p_frag[X][1][1][3]));
     };
 
-    // writes the three-term split of -m_run[qt] into the fifth k-step of Q'
-    auto publish_reference = [&](int qt) __attribute__((always_inline)) {
-        uint32_t n_hi, n_mid, n_lo;
-        split3(-m_run[qt], n_hi, n_mid, n_lo);
-        if (h == 0) {
-            q_ext[qt][1] = E::kOne | (n_hi << 16);
-            q_ext[qt][2] = n_mid | (n_lo << 16);
-        }
-    };
     // O[qt] *= f, in place.  Written as asm so that the accumulator tuples keep their registers across a
     // rarely taken branch (plain arithmetic makes the register allocator copy the 16-register tuples).
     auto scale_o = [&](int qt, float f) __attribute__((always_inline)) {
@@ -470,9 +435,10 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
             }
     };
 
-    // End of a slot.  Steady state: add the half-tile row sums.  Rare path, taken when a row sum left the
-    // safe range: the reference point of such rows moves up by a power of two, 2^shift.
-    //  - the scores of the next half-tile (buffer Y, built against the old reference) are shifted now;
+    // End of a slot.  Steady state: add the half-tile row sums.  The scores the slot built (buffer Y) are
+    // relative to m_base; rows whose reference point differs from it are corrected here (rare: it takes a
+    // wavefront whose rows differ by more than 2^64 in magnitude, or a row sum that left the safe range).
+    // When a row sum leaves the safe range the reference point of the row moves up by a power of two, 2^shift:
     //  - the row sum is rescaled now;
     //  - O is rescaled one slot later (o_pending), after the P V MFMAs of the probabilities just made,
     //    which are relative to the old reference, have been accumulated.
@@ -480,33 +446,34 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     bool any_pending = false;                  // wave-uniform
     auto finish_slot = [&](int Y, const float (&sum)[2]) __attribute__((always_inline)) {
         const bool bad = !(sum[0] <= kSumLimit) || !(sum[1] <= kSumLimit);
-        if (__any(bad) || any_pending) {
+        if (__any(bad) || any_pending || has_delta) {
             // the asm arithmetic below reads MFMA results; the compiler cannot see that, so the wait states an
             // MFMA result needs before a vector instruction may read it are spent here explicitly
             asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
             bool again = false;
 #pragma unroll
             for (int qt = 0; qt < 2; ++qt) {
-                scale_o(qt, o_pending[qt]);
+                if (any_pending) scale_o(qt, o_pending[qt]);
                 float row_sum = sum[qt];
                 asm volatile("" : "+v"(row_sum));       // keeps the arithmetic of this rare path inside the branch
                 int shift = row_sum <= kSumLimit ? 0 : max(__builtin_amdgcn_frexp_expf(row_sum) - 2, 1);
                 shift = static_cast<int>(max_across_halves(static_cast<float>(shift)));   // both half-waves of a row agree
                 const float down = __builtin_amdgcn_exp2f(static_cast<float>(-shift));
-                const float fshift = static_cast<float>(shift);
+                delta[qt] += static_cast<float>(shift);
+                m_run[qt] += static_cast<float>(shift);
+                const float d = delta[qt];
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     float t = s_acc[Y][qt][e];
-                    asm volatile("v_sub_f32 %0, %0, %1" : "+v"(t) : "v"(fshift));
+                    asm volatile("v_sub_f32 %0, %0, %1" : "+v"(t) : "v"(d));
                     s_acc[Y][qt][e] = t;
                 }
                 l_run[qt] = (l_run[qt] + row_sum) * down;
-                m_run[qt] += fshift;
-                publish_reference(qt);
                 o_pending[qt] = down;
                 again = again || __any(shift != 0);
             }
             any_pending = again;
+            has_delta = __any(delta[0] != 0.f || delta[1] != 0.f);
         } else {
             l_run[0] += sum[0];
             l_run[1] += sum[1];
@@ -535,23 +502,47 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     stage_v(1, 1);
     staged_wait(false);                // everything but this last group has landed
     __syncthreads();
-    // reference point of every row: its maximum over the first 32 keys (0 if all of them are masked)
-    score_mfma(0, 0, 0);
+    // Reference points.  Every row looks at its maximum over the first 32 keys; m_base is the largest of them in
+    // the workgroup and is folded into the bias values in LDS, so that in the steady state nothing is subtracted
+    // per score.  A row whose own maximum is more than 2^64 below m_base keeps the difference as its delta.
+    score_mfma(0, 0, 0);               // bias values in LDS are still relative to 0: plain scores
+    float row_max[2];
+    float wave_max = -INFINITY;
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
         float mx = s_acc[0][qt][0];
 #pragma unroll
         for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s_acc[0][qt][e]);
         mx = max_across_halves(mx);
-        m_run[qt] = (mx == -INFINITY || mx != mx) ? 0.f : mx;
-        publish_reference(qt);
+        row_max[qt] = (mx == -INFINITY || mx != mx) ? 0.f : mx;
+        wave_max = fmaxf(wave_max, row_max[qt]);
     }
-    score_mfma(0, 0, 0);               // the same scores, now relative to the reference
+#pragma unroll
+    for (int d = 16; d >= 1; d >>= 1) wave_max = fmaxf(wave_max, __shfl_xor(wave_max, d));
+    if (lane == 0) lds_ref[wave] = wave_max;
+    __syncthreads();                   // also: every wavefront has read the bias values of tiles 0 and 1
+    m_base = lds_ref[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) m_base = fmaxf(m_base, lds_ref[w]);
+    if (wave_u == 0) {                 // tiles 0 and 1 were converted against a base of 0
+        lds_b[0][lane] -= m_base;
+        lds_b[1][lane] -= m_base;
+    }
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+        const float gap = row_max[qt] - m_base;
+        delta[qt] = gap < -64.f ? floorf(gap) : 0.f;
+        m_run[qt] = m_base + delta[qt];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s_acc[0][qt][e] -= m_run[qt];     // the same scores, now relative to the reference
+    }
+    has_delta = __any(delta[0] != 0.f || delta[1] != 0.f);
+    __syncthreads();                   // the rebased bias values are visible
 
     for (int j = 0; j < n_tiles; ++j) {
         const int kb = j & 3, kb1 = (j + 1) & 3, kb2 = (j + 2) & 3, kb3 = (j + 3) & 3;   // stage of tile j, j+1, ..
         load_bias(j + 4, kb);          // raw bias runs one more tile ahead (converted between the slots of iteration j+2)
-        stage_k(j + 3, kb3);           // K'(j+3) replaces K'(j-1), V(j+2) replaces V(j-2): both idle since the
+        stage_k(j + 3, kb3);           // K(j+3) replaces K(j-1), V(j+2) replaces V(j-2): both idle since the
         stage_v(j + 2, kb2);           // last barrier; they are first read two barriers from now
         float sum[2];
         peek_bias(kb2);

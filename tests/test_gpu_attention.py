@@ -157,6 +157,29 @@ def test_reference_point_moves(kind):
     torch.testing.assert_close(lse.cpu(), ref_lse, atol=5e-3, rtol=1e-3)
 
 
+def test_rows_of_very_different_magnitude_in_one_workgroup():
+    """Every 7th query carries a large component along a direction in which all keys are equal, which lifts all
+    of its logits by 80 nats (115 in log2 units) without widening them: row maxima inside one workgroup then
+    differ by far more than 2^64, and the rows far below the workgroup's shared reference point keep their own
+    offset (the per-row correction path).  Same tolerance as everywhere else."""
+    L, H = 1100, 2
+    g = torch.Generator().manual_seed(11)
+    qkv = torch.randn(L, 3, H, 64, generator=g).bfloat16()
+    big = torch.zeros(L, dtype=torch.bool)
+    big[::7] = True
+    qkv[:, 1, :, 0] = 4.0
+    qkv[big, 0, :, 0] = 160.0
+    bias = torch.rand(L, generator=g).log().clamp(min=-5).bfloat16()
+    cu = _cu([L])
+    ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias)
+    out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), L, perkey_bias=bias.to(DEV),
+                                                                 return_attn_probs=True)
+    assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(lse).all())
+    _compare(out, ref)
+    torch.testing.assert_close(lse.cpu()[:, ~big], ref_lse[:, ~big], atol=5e-3, rtol=1e-3)
+    torch.testing.assert_close(lse.cpu()[:, big], ref_lse[:, big], atol=0.3, rtol=1e-3)   # 80 nats +- the 16-bit Q scaling
+
+
 def test_strided_views_and_separate_tensors():
     lens, H = [90, 41], 4
     P = sum(lens)
