@@ -36,7 +36,7 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 # WRITE_SIZE passes (KiB per dispatch), FETCH_SIZE scaled by 2.000 and WRITE_SIZE by 1.000 -- the factors a 256 MiB
 # device copy (``--only copy``) gives for the same counters.  The summaries are in profiles/.
 TRAFFIC_BYTES = {
-    "attn": int((372935 * 2.000 + 97740) * 1024),
+    "attn": int((266761 * 2.000 + 97753) * 1024),
     "merge": int((22095 * 2.000 + 25836) * 1024),
     "unmerge": int((16124 * 2.000 + 44046) * 1024),
 }
