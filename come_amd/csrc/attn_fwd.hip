@@ -149,7 +149,7 @@ __device__ inline void dma_b32(const char *base, uint32_t lane_offset, uint32_t 
 __device__ inline uint32_t lds_address(const void *p) {
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void *)(p)));
 }
-constexpr float kSumLimit = 16777216.f;      // 2^24: a tile row sum above this moves the reference point
+constexpr float kSumLimit = 1099511627776.f;  // 2^40: a half-tile row sum above this moves the reference point
 
 template <int DT, int NW>
 __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a) {
