@@ -224,17 +224,16 @@ __global__ __launch_bounds__(kThreads) void merge_vec_kernel(const MergeArgs a) 
             }
         }
 
-        if (chunk == 0) {                                   // index map and counts of this window
-            int t = 0;
-            for (int dy = 0; dy < g.gh; ++dy)
-                for (int dx = 0; dx < g.gw; ++dx, ++t)
-                    note_row(a, tok0 + static_cast<int64_t>(dy) * g.W + dx, merged ? row0 : row0 + t);
-            if (merged) {
-                note_weight(a, row0, g.G);
-            } else {
-                for (int t2 = 0; t2 < g.G; ++t2) note_weight(a, row0 + t2, 1);
-            }
+        // index map and counts of this window: token t of the window is noted by the thread of chunk t, so the
+        // few small stores go out side by side instead of one after the other from a single lane
+        const int gw_rt = GH > 0 ? GW : g.gw;
+        for (int t = chunk; t < g.G; t += chunks) {
+            const int dy = t / gw_rt;
+            const int dx = t - dy * gw_rt;
+            note_row(a, tok0 + static_cast<int64_t>(dy) * g.W + dx, merged ? row0 : row0 + t);
+            if (!merged) note_weight(a, row0 + t, 1);
         }
+        if (merged && chunk == 0) note_weight(a, row0, g.G);
         return;
     }
 
