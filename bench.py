@@ -37,8 +37,8 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 # device copy (``--only copy``) gives for the same counters.  The summaries are in profiles/.
 TRAFFIC_BYTES = {
     "attn": int((266761 * 2.000 + 97753) * 1024),
-    "merge": int((22095 * 2.000 + 25836) * 1024),
-    "unmerge": int((16124 * 2.000 + 44046) * 1024),
+    "merge": int((22066 * 2.000 + 25836) * 1024),
+    "unmerge": int((16126 * 2.000 + 44017) * 1024),
 }
 
 
