@@ -344,7 +344,12 @@ __global__ __launch_bounds__(kThreads) void split_vec_kernel(const uint4 *__rest
                                                              const IndexT *__restrict__ rev, int64_t total,
                                                              int chunks, uint4 *__restrict__ out, int64_t items,
                                                              FastDiv by_chunks) {
-    const uint32_t id = blockIdx.x * kThreads + threadIdx.x;        // items < 2^31 (checked by the host)
+    // workgroup i runs on XCD i % 8; giving every XCD one contiguous range of output rows keeps the (up to nine)
+    // consumers of a merged row on one L2
+    uint32_t bid = blockIdx.x;
+    const uint32_t per_xcd = gridDim.x >> 3;
+    if (bid < (per_xcd << 3)) bid = (bid & 7u) * per_xcd + (bid >> 3);
+    const uint32_t id = bid * kThreads + threadIdx.x;               // items < 2^31 (checked by the host)
     if (id >= items) return;
     const uint32_t quad = fast_div(id, by_chunks);
     const int chunk = static_cast<int>(id - quad * chunks);
