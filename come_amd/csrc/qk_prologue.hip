@@ -45,6 +45,8 @@ __device__ inline float group8_sum(float v) {
     return v;
 }
 
+constexpr int kRowsPerThread = 4;      // consecutive rows per lane: their loads are in flight together
+
 template <int DT>
 __global__ void __launch_bounds__(256) qk_norm_rope_kernel(const QkArgs a) {
     using V = Vec16<DT>;
@@ -53,28 +55,26 @@ __global__ void __launch_bounds__(256) qk_norm_rope_kernel(const QkArgs a) {
     const int64_t unit = gid >> 3;
     const int head = static_cast<int>(unit % a.n_heads);
     const int which = static_cast<int>((unit / a.n_heads) & 1);
-    const int64_t token = unit / (2 * a.n_heads);
-    if (token >= a.total) return;      // the eight lanes of a head leave together
+    const int64_t token0 = unit / (2 * a.n_heads) * kRowsPerThread;
+    if (token0 >= a.total) return;      // the eight lanes of a head leave together
 
-    uint4 *p = reinterpret_cast<uint4 *>(static_cast<char *>(a.ptr[which]) +
+    uint4 *p[kRowsPerThread];
+    uint4 raw[kRowsPerThread];
+    int64_t pos[kRowsPerThread];
+    bool live[kRowsPerThread];
+#pragma unroll
+    for (int t = 0; t < kRowsPerThread; ++t) {
+        live[t] = token0 + t < a.total;
+        const int64_t token = live[t] ? token0 + t : token0;
+        p[t] = reinterpret_cast<uint4 *>(static_cast<char *>(a.ptr[which]) +
                                          (token * a.row_stride[which] + head * a.head_stride[which]) * V::ELEM_BYTES) +
                lane8;
-    float f[8];
-    V::unpack(*p, f);
-
+        raw[t] = *p[t];
+        // lanes 0-3 hold the y half, lanes 4-7 the x half of a head
+        pos[t] = a.positions != nullptr ? a.positions[token * 2 + (lane8 >> 2)] : 0;
+    }
+    float g[8], b[8];
     if (a.apply_norm) {
-        float s = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) s += f[i];
-        const float mean = group8_sum(s) * (1.0f / 64.0f);
-        float q = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            f[i] -= mean;
-            q += f[i] * f[i];
-        }
-        const float rstd = rsqrtf(group8_sum(q) * (1.0f / 64.0f) + a.eps);
-        float g[8], b[8];
         if (a.gamma[which] != nullptr) {
             V::unpack(static_cast<const uint4 *>(a.gamma[which])[lane8], g);
         } else {
@@ -87,32 +87,50 @@ __global__ void __launch_bounds__(256) qk_norm_rope_kernel(const QkArgs a) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) b[i] = 0.f;
         }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) f[i] = f[i] * rstd * g[i] + b[i];
-        round_to_dtype<DT>(f);
     }
 
-    if (a.positions != nullptr) {
-        // lanes 0-3 hold the y half, lanes 4-7 the x half; lanes {0,1} and {2,3} of a half are partners
-        int64_t pos = a.positions[token * 2 + (lane8 >> 2)];
-        pos = pos < 0 ? 0 : (pos >= a.n_pos ? a.n_pos - 1 : pos);
-        const int64_t entry = (pos * 16 + (lane8 & 1) * 8) * V::ELEM_BYTES;
-        float c[8], s[8], t[8];
-        V::unpack(*reinterpret_cast<const uint4 *>(static_cast<const char *>(a.cos_table) + entry), c);
-        V::unpack(*reinterpret_cast<const uint4 *>(static_cast<const char *>(a.sin_table) + entry), s);
-        const float sign = (lane8 & 2) ? 1.f : -1.f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float partner = __shfl_xor(f[i], 2);
-            t[i] = sign * partner * s[i];
-            f[i] = f[i] * c[i];
+    for (int t = 0; t < kRowsPerThread; ++t) {
+        float f[8];
+        V::unpack(raw[t], f);
+        if (a.apply_norm) {
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s += f[i];
+            const float mean = group8_sum(s) * (1.0f / 64.0f);
+            float q = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                f[i] -= mean;
+                q += f[i] * f[i];
+            }
+            const float rstd = rsqrtf(group8_sum(q) * (1.0f / 64.0f) + a.eps);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) f[i] = f[i] * rstd * g[i] + b[i];
+            round_to_dtype<DT>(f);
         }
-        round_to_dtype<DT>(t);
-        round_to_dtype<DT>(f);
+        if (a.positions != nullptr) {
+            // lanes {0,1} and {2,3} of a half are rotation partners
+            int64_t pc = pos[t];
+            pc = pc < 0 ? 0 : (pc >= a.n_pos ? a.n_pos - 1 : pc);
+            const int64_t entry = (pc * 16 + (lane8 & 1) * 8) * V::ELEM_BYTES;
+            float c[8], sn[8], r[8];
+            V::unpack(*reinterpret_cast<const uint4 *>(static_cast<const char *>(a.cos_table) + entry), c);
+            V::unpack(*reinterpret_cast<const uint4 *>(static_cast<const char *>(a.sin_table) + entry), sn);
+            const float sign = (lane8 & 2) ? 1.f : -1.f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) f[i] += t[i];
+            for (int i = 0; i < 8; ++i) {
+                const float partner = __shfl_xor(f[i], 2);
+                r[i] = sign * partner * sn[i];
+                f[i] = f[i] * c[i];
+            }
+            round_to_dtype<DT>(r);
+            round_to_dtype<DT>(f);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) f[i] += r[i];
+        }
+        if (live[t]) *p[t] = V::pack(f);
     }
-    *p = V::pack(f);
 }
 
 }  // namespace
@@ -165,7 +183,7 @@ extern "C" int come_qk_norm_rope(void *q, void *k, int dtype,
     a.cos_table = cos_table;
     a.sin_table = sin_table;
     a.n_pos = n_pos;
-    const int64_t threads = total * 2 * n_heads * 8;
+    const int64_t threads = ceil_div(total, kRowsPerThread) * 2 * n_heads * 8;
     const int64_t blocks = ceil_div(threads, 256);
     COME_REQUIRE(blocks < (int64_t{1} << 31), COME_ERR_UNSUPPORTED, "come_qk_norm_rope: too many tokens for one launch");
     hipStream_t s = static_cast<hipStream_t>(stream);
