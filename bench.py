@@ -2,7 +2,7 @@
 
 ``python bench.py --gpus 1 --steps K --warmup W`` prints ONE JSON line.
 
-Headline ("step"): one forward pass of the biased varlen attention over the BASELINE
+Headline ("step"): one forward pass of the biased varlen attention over the benchmark
 attention configuration (16 heads x 64, two packed sequences of 25 536 and 21 848 tokens after a
 50 % / 60 % 3x3 merge of 32 frames of 37x37 patches, bias = log(count), bf16).  Its throughput is
 algorithmic flops (sum over segments of 4 L^2 d H) per second.
@@ -165,7 +165,7 @@ def jittered_frame_masks(conf, ratio, jitter, seed):
 
 
 def merge_workload(device, ratio=0.5, sets=8, frames=16, H=37, W=37, jitter=None):
-    """BASELINE merge microbench: 16 frames, 37x37 patches + 5 specials, C = 1024, bf16.  ``sets`` rotating
+    """Merge microbenchmark: 16 frames, 37x37 patches + 5 specials, C = 1024, bf16.  ``sets`` rotating
     input / output buffer sets keep the working set (> 500 MB) out of the 256 MB Infinity Cache.  With ``jitter``
     the mask comes from ``jittered_frame_masks`` instead of the joint quantile selection."""
     import torch

@@ -337,18 +337,21 @@ __global__ __launch_bounds__(kThreads) void merge_elem_kernel(const MergeArgs a)
 // ---------------------------------------------------------------------------------
 // unmerge: out[i, :] = merged[rev[i], :]
 // ---------------------------------------------------------------------------------
-constexpr int kSplitRows = 4;      // output rows per thread (independent loads in flight)
+constexpr int kSplitRows = 1;      // output rows per thread (measured best of 1, 2, 3, 4, 8)
 
 template <typename IndexT>
 __global__ __launch_bounds__(kThreads) void split_vec_kernel(const uint4 *__restrict__ merged, int64_t merged_rows,
                                                              const IndexT *__restrict__ rev, int64_t total,
                                                              int chunks, uint4 *__restrict__ out, int64_t items,
                                                              FastDiv by_chunks) {
-    // workgroup i runs on XCD i % 8; giving every XCD one contiguous range of output rows keeps the (up to nine)
+    // workgroup i runs on XCD i % 8; dealing the output rows to the XCDs in runs of 256 keeps the (up to nine)
     // consumers of a merged row on one L2
     uint32_t bid = blockIdx.x;
-    const uint32_t per_xcd = gridDim.x >> 3;
-    if (bid < (per_xcd << 3)) bid = (bid & 7u) * per_xcd + (bid >> 3);
+    constexpr uint32_t kChunk = 128;                                 // consecutive workgroups (256 output rows) that stay on one XCD
+    if (kChunk > 0 && bid < (gridDim.x / (8u * kChunk)) * (8u * kChunk)) {
+        const uint32_t local = bid >> 3;
+        bid = ((local / kChunk) * 8u + (bid & 7u)) * kChunk + local % kChunk;
+    }
     const uint32_t id = bid * kThreads + threadIdx.x;               // items < 2^31 (checked by the host)
     if (id >= items) return;
     const uint32_t quad = fast_div(id, by_chunks);

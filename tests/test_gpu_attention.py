@@ -236,7 +236,7 @@ def test_unsupported_arguments_raise():
 
 
 def test_full_size_c3_rows_against_oracle_rows():
-    """BASELINE attention config: 16 heads x 64, two packed sequences of 25 536 and 21 848 tokens,
+    """Benchmark attention configuration: 16 heads x 64, two packed sequences of 25 536 and 21 848 tokens,
     bias = log(count), count in {1, 9}.  The full fp32 oracle is too slow on a CPU at this size, so a
     sample of query rows is checked against the closed form, plus the logsumexp identity."""
     H, D = 16, 64

@@ -150,7 +150,7 @@ def test_int32_index_map_and_counts_and_split():
 
 
 def test_full_size_c2_properties():
-    # BASELINE merge microbench shape: 16 frames of 37x37 (+5 specials), C = 1024, bf16
+    # merge microbenchmark shape: 16 frames of 37x37 (+5 specials), C = 1024, bf16
     B, H, W, S, C = 16, 37, 37, 5, 1024
     g = torch.Generator().manual_seed(0)
     tokens = torch.randn(B, S + H * W, C, generator=g).bfloat16().to(DEV)
