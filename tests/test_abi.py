@@ -53,3 +53,30 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libcome_hip.so")
     with pytest.raises(RuntimeError, match="no fallback"):
         _lib.load()
+
+
+def test_header_is_plain_c_and_links_against_the_library(tmp_path):
+    """The header compiles as C99 and a C caller that references every declared function links against the
+    shared library (no C++ names, no torch types)."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("gcc not available")
+    names = _declared_functions()
+    src = tmp_path / "caller.c"
+    body = "\n".join(f"    table[{i}] = (fn)&{name};" for i, name in enumerate(names))
+    src.write_text('#include "come_hip.h"\n#include <stdio.h>\ntypedef void (*fn)(void);\nint main(void) {\n'
+                   f"    fn table[{len(names)}];\n{body}\n"
+                   '    printf("%d %s|\\n", come_version(), come_last_error());\n'
+                   f"    return table[0] == 0;\n}}\n")
+    exe = tmp_path / "caller"
+    lib_dir = os.path.dirname(_lib.LIB_PATH)
+    cmd = [gcc, "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe),
+           "-L", lib_dir, "-lcome_hip", f"-Wl,-rpath,{lib_dir}", "-Wl,--allow-shlib-undefined"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+    run = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert run.returncode == 0, run.stderr
+    assert run.stdout.startswith(str(_lib.load().come_version()))
