@@ -613,6 +613,9 @@ extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v,
     COME_REQUIRE(softmax_scale > 0.f && softmax_scale < INFINITY, COME_ERR_INVALID,
                  "come_attn_varlen_fwd: softmax_scale must be positive and finite");
     if (total == 0 || max_seqlen == 0) return COME_OK;
+    // offsets inside a segment are 32-bit byte offsets from the segment's first row
+    COME_REQUIRE(max_seqlen * (k_row_stride > v_row_stride ? k_row_stride : v_row_stride) * 2 < (1ll << 32),
+                 COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: a segment may span at most 4 GiB of K or V rows");
     COME_REQUIRE(q && k && v && out && cu_seqlens, COME_ERR_INVALID, "come_attn_varlen_fwd: NULL tensor");
     const int64_t strides[8] = {q_row_stride, q_head_stride, k_row_stride, k_head_stride,
                                 v_row_stride, v_head_stride, o_row_stride, o_head_stride};

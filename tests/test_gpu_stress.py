@@ -93,3 +93,24 @@ def test_frame_and_global_attention_sampled():
         diff = (out[row] - ref).abs()
         assert float(diff.max()) <= 1e-2 and float(diff.mean()) <= 1e-3
         torch.testing.assert_close(lse[:, row], torch.logsumexp(scores, -1), atol=2e-3, rtol=1e-3)
+
+
+def test_unmerged_global_segment_of_133k_tokens_sampled():
+    """The unmerged stress sequence as one segment (133 248 tokens, row stride 768 B -> 102 MB of packed q/k/v):
+    exercises the large offsets; sampled rows against the closed form (2 heads keep it at 9 TFLOP)."""
+    Hh, D, L = 2, 64, FRAMES * N
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn(L, 3, Hh, D, generator=g).bfloat16()
+    bias = (torch.rand(L, generator=g) * 2).bfloat16()
+    cu = torch.tensor([0, L], dtype=torch.int32)
+    out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), L, perkey_bias=bias.to(DEV),
+                                                                 softmax_scale=0.125, return_attn_probs=True)
+    out, lse = out.float().cpu(), lse.cpu()
+    assert bool(torch.isfinite(out).all())
+    q, k, v = qkv.float().unbind(1)
+    for row in [0, 255, 256, 511, 512, 70000, L - 513, L - 1]:
+        scores = torch.einsum("hd,khd->hk", q[row], k) * 0.125 + bias.float()[None]
+        ref = torch.einsum("hk,khd->hd", torch.softmax(scores, -1), v)
+        diff = (out[row] - ref).abs()
+        assert float(diff.max()) <= 1e-2 and float(diff.mean()) <= 1e-3
+        torch.testing.assert_close(lse[:, row], torch.logsumexp(scores, -1), atol=2e-3, rtol=1e-3)
