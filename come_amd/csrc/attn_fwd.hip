@@ -539,6 +539,18 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     has_delta = __any(delta[0] != 0.f || delta[1] != 0.f);
     __syncthreads();                   // the rebased bias values are visible
 
+    // A wavefront whose 64 queries all lie beyond the end of the segment (last workgroup of a segment) only
+    // helps with the staging: it has nothing to compute and nothing to write.  Wavefront 0 always has queries.
+    if (q0 + wave_u * 64 >= L) {
+        for (int j = 0; j < n_tiles; ++j) {
+            stage_k(j + 3, (j + 3) & 3);
+            stage_v(j + 2, (j + 2) & 3);
+            staged_wait(true);
+            __syncthreads();
+        }
+        return;
+    }
+
     for (int j = 0; j < n_tiles; ++j) {
         const int kb = j & 3, kb1 = (j + 1) & 3, kb2 = (j + 2) & 3, kb3 = (j + 3) & 3;   // stage of tile j, j+1, ..
         load_bias(j + 4, kb);          // raw bias runs one more tile ahead (converted between the slots of iteration j+2)
