@@ -28,13 +28,55 @@ constexpr int kKeysPerThread = 8;      // means kept in registers up to 8 * 1024
 
 // k-th smallest (0-based) of the n values the workgroup holds: thread t owns values t, t + 1024, ...
 // either in mine[] (n <= 8192) or in vals[] (global).  All threads call it and all receive the answer.
-// hist: 256 counters, ctl: 2 words of LDS.
+// hist: 256 counters, ctl: 2 words, red: 34 words of LDS.
+// The leading bits that the smallest and the largest key share are decided up front, so the first 8-bit digit
+// already spreads the keys over the histogram (confidence means sit in a narrow range: without this step they
+// would all hit the same few counters) and narrow ranges need fewer passes.
 __device__ float radix_select(const float *vals, const float *mine, bool in_regs, int n, int k, uint32_t *hist,
-                              uint32_t *ctl) {
-    uint32_t prefix = 0, fixed = 0;
+                              uint32_t *ctl, uint32_t *red) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    for (int shift = 24; shift >= 0; shift -= 8) {
+    uint32_t kmin = 0xffffffffu, kmax = 0u;
+    if (in_regs) {
+#pragma unroll
+        for (int r = 0; r < kKeysPerThread; ++r) {
+            if (static_cast<int>(threadIdx.x) + r * kSelectThreads < n) {
+                const uint32_t key = ordered_key(mine[r]);
+                kmin = min(kmin, key);
+                kmax = max(kmax, key);
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < n; i += blockDim.x) {
+            const uint32_t key = ordered_key(vals[i]);
+            kmin = min(kmin, key);
+            kmax = max(kmax, key);
+        }
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        kmin = min(kmin, static_cast<uint32_t>(__shfl_xor(static_cast<int>(kmin), d)));
+        kmax = max(kmax, static_cast<uint32_t>(__shfl_xor(static_cast<int>(kmax), d)));
+    }
+    if (lane == 0) {
+        red[wave] = kmin;
+        red[16 + wave] = kmax;
+    }
+    __syncthreads();
+    kmin = red[0];
+    kmax = red[16];
+#pragma unroll
+    for (int w = 1; w < kSelectThreads / 64; ++w) {
+        kmin = min(kmin, red[w]);
+        kmax = max(kmax, red[16 + w]);
+    }
+    int open_bits = 32 - __clz(static_cast<int>(kmin ^ kmax));        // low bits in which keys differ (0: all equal)
+    if (kmin == kmax) open_bits = 0;
+    uint32_t fixed = open_bits >= 32 ? 0u : ~((1u << open_bits) - 1u);
+    uint32_t prefix = kmin & fixed;
+    int shift = open_bits;
+    while (shift > 0) {
+        shift = shift > 8 ? shift - 8 : 0;
         if (threadIdx.x < 256) hist[threadIdx.x] = 0;
         __syncthreads();
         if (in_regs) {
@@ -80,11 +122,12 @@ __device__ float radix_select(const float *vals, const float *mine, bool in_regs
             }
         }
         __syncthreads();
+        // a digit may overlap bits that are already decided (last pass): they agree by construction
         prefix |= ctl[0] << shift;
         fixed |= 255u << shift;
         k = static_cast<int>(ctl[1]);
     }
-    __syncthreads();                       // ctl and hist are free again
+    __syncthreads();                       // ctl, hist and red are free again
     return key_to_float(prefix);
 }
 
@@ -118,7 +161,7 @@ __global__ __launch_bounds__(kSelectThreads) void select_windows_kernel(
     using V = Vec16<DT>;
     __shared__ uint32_t hist[256];
     __shared__ uint32_t ctl[2];
-    __shared__ float red[17];
+    __shared__ float red[34];
 
     const int mh = H / gh, mw = W / gw;
     const int M = mh * mw;
@@ -186,7 +229,7 @@ __global__ __launch_bounds__(kSelectThreads) void select_windows_kernel(
     //    the upper one is either the same value again (duplicates) or the smallest value above the lower one.
     float cut = threshold;
     if (mode == 0) {
-        const float a = radix_select(my_means, mine, in_regs, n, rank_lo, hist, ctl);
+        const float a = radix_select(my_means, mine, in_regs, n, rank_lo, hist, ctl, reinterpret_cast<uint32_t *>(red));
         float b = a;
         if (rank_hi != rank_lo) {
             float le = 0.f;                                   // exact in fp32: n < 2^24
