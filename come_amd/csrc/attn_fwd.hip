@@ -57,6 +57,7 @@ template <> struct Elem<COME_BF16> {
     __device__ static inline float to_f32(uint16_t x) { return __uint_as_float(static_cast<uint32_t>(x) << 16); }
     __device__ static inline uint16_t from_f32(float x) { return static_cast<uint16_t>(pack2_bf16(x, 0.f) & 0xffffu); }
     __device__ static inline uint32_t pack2(float lo, float hi) { return pack2_bf16(lo, hi); }
+    __device__ static inline uint32_t pack2_prob(float lo, float hi) { return pack2_bf16(lo, hi); }
     // acc + lo(w) + hi(w) with fp32 accumulation (v_dot2c_f32_bf16 against packed ones)
     __device__ static inline float dot2_ones(uint32_t w, float acc) {
         return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(come_bf16x2, w),
@@ -71,6 +72,11 @@ template <> struct Elem<COME_F16> {
     __device__ static inline float to_f32(uint16_t x) { return __half2float(__builtin_bit_cast(__half, x)); }
     __device__ static inline uint16_t from_f32(float x) { return __builtin_bit_cast(uint16_t, __float2half_rn(x)); }
     __device__ static inline uint32_t pack2(float lo, float hi) { return pack2_f16(lo, hi); }
+    // probabilities: round toward zero, so that a value beyond the fp16 range saturates at 65504 instead of
+    // becoming infinite (row sums are taken from the converted values, so numerator and denominator agree)
+    __device__ static inline uint32_t pack2_prob(float lo, float hi) {
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+    }
     __device__ static inline float dot2_ones(uint32_t w, float acc) {
         return __builtin_amdgcn_fdot2(__builtin_bit_cast(come_f16x2, w),
                                       __builtin_bit_cast(come_f16x2, kOne | (kOne << 16)), acc, false);
@@ -149,11 +155,24 @@ __device__ inline void dma_b32(const char *base, uint32_t lane_offset, uint32_t 
 __device__ inline uint32_t lds_address(const void *p) {
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void *)(p)));
 }
-constexpr float kSumLimit = 1099511627776.f;  // 2^40: a half-tile row sum above this moves the reference point
+// Range of the probabilities relative to the reference point of their row.  They are stored in the 16-bit type of
+// the inputs: bf16 has the exponent range of fp32, fp16 reaches only 65504 and loses precision below 2^-14.
+//   kSumLimit  a half-tile row sum above this moves the reference point of the row up
+//   kMaxGap    a row whose own maximum lies further below the workgroup's reference point keeps its own offset
+template <int DT> struct Range;
+template <> struct Range<COME_BF16> {
+    static constexpr float kSumLimit = 1099511627776.f;   // 2^40
+    static constexpr float kMaxGap = 64.f;
+};
+template <> struct Range<COME_F16> {
+    static constexpr float kSumLimit = 32.f;               // 2^5: a probability may grow by 2^11 more before fp16 saturates
+    static constexpr float kMaxGap = 4.f;
+};
 
 template <int DT, int NW>
 __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a) {
     using E = Elem<DT>;
+    constexpr float kSumLimit = Range<DT>::kSumLimit;
     static_assert(NW == 4 || NW == 8, "4 or 8 wavefronts per workgroup");
     constexpr int kBlockM = 64 * NW;           // queries per workgroup
     constexpr int kThreads = 64 * NW;
@@ -402,7 +421,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
             }
             if (c > 0) {                    // pack and add the pair whose exponentials were issued one chunk ago
                 const int pc = c - 1, qt = pc >> 3, w = pc & 7;
-                const uint32_t pw = E::pack2(p0, p1);
+                const uint32_t pw = E::pack2_prob(p0, p1);
                 p_frag[X][qt][w >> 2][w & 3] = pw;
                 sum[qt] = E::dot2_ones(pw, sum[qt]);
             }
@@ -413,7 +432,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
             __builtin_amdgcn_sched_barrier(0);
         }
         {
-            const uint32_t pw = E::pack2(p0, p1);
+            const uint32_t pw = E::pack2_prob(p0, p1);
             p_frag[X][1][1][3] = pw;
             sum[1] = E::dot2_ones(pw, sum[1]);
         }
@@ -437,7 +456,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
 
     // End of a slot.  Steady state: add the half-tile row sums.  The scores the slot built (buffer Y) are
     // relative to m_base; rows whose reference point differs from it are corrected here (rare: it takes a
-    // wavefront whose rows differ by more than 2^64 in magnitude, or a row sum that left the safe range).
+    // wavefront whose rows differ by more than 2^kMaxGap in magnitude, or a row sum that left the safe range).
     // When a row sum leaves the safe range the reference point of the row moves up by a power of two, 2^shift:
     //  - the row sum is rescaled now;
     //  - O is rescaled one slot later (o_pending), after the P V MFMAs of the probabilities just made,
@@ -504,7 +523,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     __syncthreads();
     // Reference points.  Every row looks at its maximum over the first 32 keys; m_base is the largest of them in
     // the workgroup and is folded into the bias values in LDS, so that in the steady state nothing is subtracted
-    // per score.  A row whose own maximum is more than 2^64 below m_base keeps the difference as its delta.
+    // per score.  A row whose own maximum is more than 2^kMaxGap below m_base keeps the difference as its delta.
     score_mfma(0, 0, 0);               // bias values in LDS are still relative to 0: plain scores
     float row_max[2];
     float wave_max = -INFINITY;
@@ -531,7 +550,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
         const float gap = row_max[qt] - m_base;
-        delta[qt] = gap < -64.f ? floorf(gap) : 0.f;
+        delta[qt] = gap < -Range<DT>::kMaxGap ? floorf(gap) : 0.f;
         m_run[qt] = m_base + delta[qt];
 #pragma unroll
         for (int e = 0; e < 16; ++e) s_acc[0][qt][e] -= m_run[qt];     // the same scores, now relative to the reference

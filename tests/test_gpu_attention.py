@@ -157,6 +157,24 @@ def test_reference_point_moves(kind):
     torch.testing.assert_close(lse.cpu(), ref_lse, atol=5e-3, rtol=1e-3)
 
 
+def test_fp16_reference_point_moves_within_its_narrow_range():
+    """fp16 stores the probabilities in fp16, so its reference points move much earlier (row sums above 2^5, rows
+    more than 2^4 below the workgroup's reference keep their own offset).  A slowly rising bias (20 nats over the
+    segment) and rows of different scale exercise both paths inside the range fp16 can hold."""
+    L, H = 1500, 2
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn(L, 3, H, 64, generator=g).half()
+    qkv[::3, 0] = (qkv[::3, 0].float() * 2).half()
+    bias = torch.linspace(-10.0, 10.0, L).half()
+    cu = _cu([L])
+    ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias)
+    out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), L, perkey_bias=bias.to(DEV),
+                                                                 return_attn_probs=True)
+    assert bool(torch.isfinite(out).all())
+    _compare(out, ref)
+    torch.testing.assert_close(lse.cpu(), ref_lse, atol=5e-3, rtol=1e-3)
+
+
 def test_rows_of_very_different_magnitude_in_one_workgroup():
     """Every 7th query carries a large component along a direction in which all keys are equal, which lifts all
     of its logits by 80 nats (115 in log2 units) without widening them: row maxima inside one workgroup then
