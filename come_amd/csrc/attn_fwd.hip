@@ -49,7 +49,15 @@ struct AttnArgs {
     int64_t total;
     int n_heads, n_mblocks, n_units;
     float scale_log2;
+    // key-split tail: the last nb_tail query blocks of every (segment, head) unit are computed by `splits`
+    // workgroups each, every one over its share of the keys, into `work`; a second kernel combines them
+    int nb_tail, splits;
+    int64_t n_full_wg;               // workgroups in front of the split ones
+    float *work;
 };
+
+constexpr int kPieceExtra = 2;       // per query row of a piece: 64 unnormalised outputs, reference point, row sum
+
 
 template <int DT> struct Elem;
 template <> struct Elem<COME_BF16> {
@@ -108,11 +116,28 @@ __device__ inline s16x4 lds_read_tr(const uint16_t *p) {
 // i % 8, each XCD with its own L2: the query blocks of one (segment, head) unit run back to back
 // on one XCD and share that unit's K/V there, and units are dealt to the XCDs round-robin so that
 // segments of different lengths spread evenly.  The grid is padded to 8 * ceil(units / 8) units.
-__device__ inline bool locate_block(const AttnArgs &a, int &mblk, int &head, int &seq) {
-    const int xcd = blockIdx.x & 7;
-    const int local = blockIdx.x >> 3;
-    const int unit = xcd + 8 * (local / a.n_mblocks);
-    mblk = local % a.n_mblocks;
+// A split workgroup (behind the n_full_wg ordinary ones) gets the index of its query block among the unit's
+// tail blocks (tail >= 0) and its key share ks; the pieces of one query block are neighbours on one XCD.
+__device__ inline bool locate_block(const AttnArgs &a, int &mblk, int &head, int &seq, int &tail, int &ks) {
+    int unit;
+    if (static_cast<int64_t>(blockIdx.x) < a.n_full_wg) {
+        const int xcd = blockIdx.x & 7;
+        const int local = blockIdx.x >> 3;
+        unit = xcd + 8 * (local / a.n_mblocks);
+        mblk = local % a.n_mblocks;
+        tail = -1;
+        ks = 0;
+    } else {
+        const int e = static_cast<int>(blockIdx.x - a.n_full_wg);
+        const int xcd = e & 7;
+        const int local = e >> 3;
+        const int per_unit = a.nb_tail * a.splits;
+        unit = xcd + 8 * (local / per_unit);
+        const int within = local % per_unit;
+        tail = within / a.splits;
+        ks = within % a.splits;
+        mblk = 0;
+    }
     head = unit % a.n_heads;
     seq = unit / a.n_heads;
     return unit < a.n_units;
@@ -187,12 +212,28 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     __shared__ __attribute__((aligned(256))) uint32_t lds_braw[kStages][kBlockN];   // raw bias words as loaded
     __shared__ float lds_ref[NW];                                                   // prologue: reference point per wavefront
 
-    int mblk, head, seq;
-    if (!locate_block(a, mblk, head, seq)) return;
+    int mblk, head, seq, tail, ks;
+    if (!locate_block(a, mblk, head, seq, tail, ks)) return;
     const int seq_start = a.cu[seq];
     const int L = a.cu[seq + 1] - seq_start;
+    const int n_qblocks = (L + kBlockM - 1) / kBlockM;
+    if (tail >= 0) {
+        mblk = n_qblocks - a.nb_tail + tail;          // split workgroup: one of the unit's last query blocks
+        if (mblk < 0) return;
+    } else if (a.splits > 1 && mblk >= n_qblocks - a.nb_tail) {
+        return;                                       // left to the split workgroups (or beyond the segment)
+    }
     const int q0 = mblk * kBlockM;
     if (q0 >= L) return;
+    // keys of this workgroup: all tiles, or share ks of them
+    const int all_tiles = (L + kBlockN - 1) / kBlockN;
+    const int tile_base = tail >= 0 ? static_cast<int>(static_cast<int64_t>(ks) * all_tiles / a.splits) : 0;
+    const int tile_end = tail >= 0 ? static_cast<int>(static_cast<int64_t>(ks + 1) * all_tiles / a.splits) : all_tiles;
+    float *piece = nullptr;
+    if (tail >= 0) {
+        const int64_t index = (static_cast<int64_t>(seq * a.n_heads + head) * a.nb_tail + tail) * a.splits + ks;
+        piece = a.work + index * (kBlockM * (kHeadDim + kPieceExtra));
+    }
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -241,7 +282,8 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     const uint32_t k_last = static_cast<uint32_t>(L - 1) * k_rs_b, v_last = static_cast<uint32_t>(L - 1) * v_rs_b;
     const uint32_t k_tile_step = static_cast<uint32_t>(kBlockN) * k_rs_b, v_tile_step = static_cast<uint32_t>(kBlockN) * v_rs_b;
 
-    auto stage_k = [&](int tile, int buf) __attribute__((always_inline)) {
+    auto stage_k = [&](int rel_tile, int buf) __attribute__((always_inline)) {
+        const int tile = tile_base + rel_tile;
         const int n0 = tile * kBlockN;
         const uint32_t tile_off = static_cast<uint32_t>(tile) * k_tile_step;         // wave-uniform
         const bool full = n0 + kBlockN <= L;                                        // wave-uniform
@@ -254,13 +296,15 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     };
     // raw bias of the 64 keys of a tile: wavefront 0 brings the aligned 32-bit word that holds each key's
     // 16-bit bias; it is converted to a float two iterations later (commit_bias)
-    auto load_bias = [&](int tile, int buf) __attribute__((always_inline)) {
+    auto load_bias = [&](int rel_tile, int buf) __attribute__((always_inline)) {
+        const int tile = tile_base + rel_tile;
         if (wave_u == 0 && b_seg) {
             const uint32_t key = static_cast<uint32_t>(min(tile * kBlockN + lane, L - 1));
             dma_b32(b_seg, ((b_mis + 2u * key) & ~3u), lds_address(&lds_braw[buf][0]));
         }
     };
-    auto stage_v = [&](int tile, int buf) __attribute__((always_inline)) {
+    auto stage_v = [&](int rel_tile, int buf) __attribute__((always_inline)) {
+        const int tile = tile_base + rel_tile;
         const int n0 = tile * kBlockN;
         const uint32_t tile_off = static_cast<uint32_t>(tile) * v_tile_step;
         const bool full = n0 + kBlockN <= L;
@@ -278,9 +322,9 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     auto peek_bias = [&](int buf) __attribute__((always_inline)) {
         if (wave_u == 0 && b_seg) b_word = lds_braw[buf][lane];
     };
-    auto commit_bias = [&](int tile, int buf) __attribute__((always_inline)) {
+    auto commit_bias = [&](int rel_tile, int buf) __attribute__((always_inline)) {
         if (wave_u == 0) {
-            const int key = tile * kBlockN + lane;
+            const int key = (tile_base + rel_tile) * kBlockN + lane;
             float bias = 0.f;
             if (b_seg) {
                 const uint32_t at = b_mis + 2u * static_cast<uint32_t>(min(key, L - 1));
@@ -500,7 +544,14 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     };
 
     // ---- prologue
-    const int n_tiles = (L + kBlockN - 1) / kBlockN;
+    const int n_tiles = tile_end - tile_base;
+    if (n_tiles <= 0) {                      // a key share without tiles (segment shorter than the split count)
+        for (int i = tid; i < kBlockM; i += kThreads) {
+            piece[kBlockM * kHeadDim + i] = -1e30f;               // reference point
+            piece[kBlockM * (kHeadDim + 1) + i] = 0.f;            // row sum
+        }
+        return;
+    }
     {   // the last V stage stands in for "tile -1": zeros (its probabilities are zero as well)
         u32x4 *z = reinterpret_cast<u32x4 *>(&lds_v[kStages - 1][0]);
         for (int i = tid; i < kBlockN * kHeadDim / 8; i += kThreads) z[i] = zero4();
@@ -596,6 +647,30 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
 #pragma unroll
             for (int e = 0; e < 16; ++e) o_acc[qt][dt][e] *= o_pending[qt];
 
+    // ---- epilogue of a split workgroup: unnormalised outputs, reference point and row sum of its key share
+    if (piece != nullptr) {
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+            const float l_tot = sum_across_halves(l_run[qt]);
+            const int local_row = (wave * 2 + qt) * 32 + r;
+            if (q0 + local_row < L) {
+                float *op = piece + local_row * kHeadDim + 4 * h;
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                        *reinterpret_cast<f32x4 *>(op + 32 * dt + 8 * g) =
+                            f32x4{o_acc[qt][dt][4 * g], o_acc[qt][dt][4 * g + 1], o_acc[qt][dt][4 * g + 2],
+                                  o_acc[qt][dt][4 * g + 3]};
+                if (h == 0) {
+                    piece[kBlockM * kHeadDim + local_row] = m_run[qt];
+                    piece[kBlockM * (kHeadDim + 1) + local_row] = l_tot;
+                }
+            }
+        }
+        return;
+    }
+
     // ---- epilogue: normalise, write O (and LSE)
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
@@ -620,17 +695,130 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     }
 }
 
+// Combines the key shares of the split query blocks: with m* the largest reference point of a row,
+// O = sum_i 2^(m_i - m*) O_i / sum_i 2^(m_i - m*) l_i.  One workgroup per split query block.
+template <int DT>
+__global__ __launch_bounds__(256) void attn_combine_kernel(const AttnArgs a, int block_m) {
+    using E = Elem<DT>;
+    const int tail = blockIdx.x % a.nb_tail;
+    const int unit = blockIdx.x / a.nb_tail;
+    const int head = unit % a.n_heads;
+    const int seq = unit / a.n_heads;
+    const int seq_start = a.cu[seq];
+    const int L = a.cu[seq + 1] - seq_start;
+    const int mblk = (L + block_m - 1) / block_m - a.nb_tail + tail;
+    if (mblk < 0) return;
+    const int q0 = mblk * block_m;
+    const int64_t piece_floats = static_cast<int64_t>(block_m) * (kHeadDim + kPieceExtra);
+    const float *first = a.work + (static_cast<int64_t>(unit) * a.nb_tail + tail) * a.splits * piece_floats;
+    for (int idx = threadIdx.x; idx < block_m * (kHeadDim / 4); idx += blockDim.x) {
+        const int local_row = idx / (kHeadDim / 4);
+        const int c4 = idx % (kHeadDim / 4);
+        if (q0 + local_row >= L) continue;
+        float m_star = -INFINITY;
+        for (int i = 0; i < a.splits; ++i) {
+            const float *pc = first + i * piece_floats;
+            if (pc[block_m * (kHeadDim + 1) + local_row] > 0.f) m_star = fmaxf(m_star, pc[block_m * kHeadDim + local_row]);
+        }
+        float l_sum = 0.f;
+        f32x4 o = {0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < a.splits; ++i) {
+            const float *pc = first + i * piece_floats;
+            const float l_i = pc[block_m * (kHeadDim + 1) + local_row];
+            if (!(l_i > 0.f)) continue;
+            const float w = __builtin_amdgcn_exp2f(pc[block_m * kHeadDim + local_row] - m_star);
+            l_sum += w * l_i;
+            const f32x4 v = *reinterpret_cast<const f32x4 *>(pc + local_row * kHeadDim + 4 * c4);
+            o += v * w;
+        }
+        const float inv = 1.0f / l_sum;
+        u32x2 packed;
+        packed[0] = E::pack2(o[0] * inv, o[1] * inv);
+        packed[1] = E::pack2(o[2] * inv, o[3] * inv);
+        *reinterpret_cast<u32x2 *>(a.out + static_cast<int64_t>(seq_start + q0 + local_row) * a.o_rs + head * a.o_hs + 4 * c4) = packed;
+        if (c4 == 0 && a.lse)
+            a.lse[static_cast<int64_t>(head) * a.total + seq_start + q0 + local_row] =
+                (m_star + __log2f(l_sum)) * 0.6931471805599453f;
+    }
+}
+
+// How a launch is shaped.
+//  - 8 wavefronts per workgroup share every staged K / V tile among 512 queries (half the L2 -> LDS traffic),
+//    but such a workgroup fills a whole CU, so a partly filled last round of workgroups costs a full round.
+//    Without a work buffer it is used for long segments only when the expected number of workgroups nearly
+//    fills its last round; otherwise two 256-query workgroups share a CU and the last round finishes early.
+//  - With a work buffer the query blocks of that last round are cut along the keys into `splits` workgroups
+//    each, which fill the chip with short pieces instead; a small kernel combines the pieces.
+struct Plan {
+    bool wide = false;
+    int nb_tail = 0, splits = 1;
+    int64_t work_bytes = 0;
+};
+
+int cu_count() {
+    static const int n_cu = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        return n;
+    }();
+    return n_cu;
+}
+
+Plan make_plan(int64_t n_seq, int64_t total, int64_t n_heads, int64_t max_seqlen, bool may_split) {
+    Plan p;
+    if (max_seqlen < 4096) return p;
+    const int n_cu = cu_count();
+    const int64_t units = n_seq * n_heads;
+    // one segment: exact; several: half a block of padding per segment on average
+    const int64_t expected = n_seq == 1 ? n_heads * ceil_div(total, 512) : n_heads * ceil_div(total + n_seq * 256, 512);
+    const int64_t rounds = ceil_div(expected, n_cu);
+    if (expected * 100 >= rounds * n_cu * 95) {
+        p.wide = true;
+        return p;
+    }
+    if (!may_split) return p;
+    const int64_t full = expected / n_cu;
+    const int64_t tail = expected - full * n_cu;
+    if (full == 0 || tail == 0) return p;
+    const int64_t nb_tail = ceil_div(tail, units);
+    const int64_t tiles = ceil_div(max_seqlen, kBlockN);
+    int best = 0;
+    double best_cost = 0.6;                          // what the partly filled last round of 256-query workgroups costs
+    for (int sp = 2; sp <= 8; ++sp) {
+        if (tiles / sp < 16) break;                  // pieces of at least 16 key tiles
+        const double cost = static_cast<double>(ceil_div(nb_tail * units * sp, n_cu)) / sp + 0.02 * sp;
+        if (cost < best_cost) {
+            best_cost = cost;
+            best = sp;
+        }
+    }
+    if (best == 0 || nb_tail > ceil_div(max_seqlen, 512)) return p;
+    p.wide = true;
+    p.nb_tail = static_cast<int>(nb_tail);
+    p.splits = best;
+    p.work_bytes = units * nb_tail * best * 512 * (kHeadDim + kPieceExtra) * static_cast<int64_t>(sizeof(float));
+    return p;
+}
+
 }  // namespace
 }  // namespace come
 
 using namespace come;
 
-extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v, int dtype, int64_t q_row_stride,
-                                    int64_t q_head_stride, int64_t k_row_stride, int64_t k_head_stride,
-                                    int64_t v_row_stride, int64_t v_head_stride, const int32_t *cu_seqlens,
-                                    int64_t n_seq, int64_t total, int64_t n_heads, int64_t head_dim,
-                                    const void *perkey_bias, int64_t max_seqlen, float softmax_scale, void *out,
-                                    int64_t o_row_stride, int64_t o_head_stride, float *lse, void *stream) {
+extern "C" int64_t come_attn_work_bytes(int64_t n_seq, int64_t total, int64_t n_heads, int64_t max_seqlen) {
+    if (n_seq <= 0 || total <= 0 || n_heads <= 0 || max_seqlen <= 0) return 0;
+    return make_plan(n_seq, total, n_heads, max_seqlen, true).work_bytes;
+}
+
+extern "C" int come_attn_varlen_fwd_ws(const void *q, const void *k, const void *v, int dtype, int64_t q_row_stride,
+                                       int64_t q_head_stride, int64_t k_row_stride, int64_t k_head_stride,
+                                       int64_t v_row_stride, int64_t v_head_stride, const int32_t *cu_seqlens,
+                                       int64_t n_seq, int64_t total, int64_t n_heads, int64_t head_dim,
+                                       const void *perkey_bias, int64_t max_seqlen, float softmax_scale, void *out,
+                                       int64_t o_row_stride, int64_t o_head_stride, float *lse, void *work,
+                                       int64_t work_bytes, void *stream) {
     clear_error();
     COME_REQUIRE(dtype == COME_BF16 || dtype == COME_F16, COME_ERR_UNSUPPORTED,
                  "come_attn_varlen_fwd: only fp16 and bf16 are supported");
@@ -662,23 +850,10 @@ extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v,
                      (reinterpret_cast<uintptr_t>(v) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0,
                  COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: q/k/v must be 16-byte aligned, out 8-byte aligned");
 
-    // 8 wavefronts per workgroup share every staged K / V tile among 512 queries (half the L2 -> LDS traffic),
-    // but such a workgroup fills a whole CU, so a partly filled last round of workgroups costs a full round.
-    // It is used for long segments when the expected number of workgroups nearly fills its last round;
-    // otherwise two 256-query workgroups share a CU and the last round finishes early on the CUs it uses.
-    bool wide = false;
-    if (max_seqlen >= 4096) {
-        static const int n_cu = [] {
-            int dev = 0, n = 0;
-            if (hipGetDevice(&dev) != hipSuccess ||
-                hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-                n = 256;
-            return n;
-        }();
-        const int64_t expected = n_heads * ceil_div(total + n_seq * 256, 512);
-        const int64_t rounds = ceil_div(expected, n_cu);
-        wide = expected * 100 >= rounds * n_cu * 95;
-    }
+    Plan plan = make_plan(n_seq, total, n_heads, max_seqlen, work != nullptr);
+    if (plan.splits > 1 && (work_bytes < plan.work_bytes || (reinterpret_cast<uintptr_t>(work) & 15) != 0))
+        plan = make_plan(n_seq, total, n_heads, max_seqlen, false);        // buffer too small or misaligned: no split
+    const bool wide = plan.wide;
     const int kBlockM = wide ? 512 : 256;
     AttnArgs a{};
     a.q = static_cast<const uint16_t *>(q);
@@ -697,7 +872,11 @@ extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v,
     a.n_mblocks = static_cast<int>(ceil_div(max_seqlen, kBlockM));
     a.scale_log2 = softmax_scale * 1.4426950408889634f;
     a.n_units = static_cast<int>(n_seq * n_heads);
-    const int64_t n_wg = ceil_div(n_seq * n_heads, 8) * 8 * a.n_mblocks;
+    a.nb_tail = plan.nb_tail;
+    a.splits = plan.splits;
+    a.work = static_cast<float *>(work);
+    a.n_full_wg = ceil_div(n_seq * n_heads, 8) * 8 * a.n_mblocks;
+    const int64_t n_wg = a.n_full_wg + ceil_div(n_seq * n_heads, 8) * 8 * (plan.splits > 1 ? plan.nb_tail * plan.splits : 0);
     COME_REQUIRE(n_wg < (1ll << 31), COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: grid too large");
     const dim3 grid(static_cast<unsigned>(n_wg)), block(wide ? 512 : 256);
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -709,5 +888,23 @@ extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v,
         else hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_F16, 4>), grid, block, 0, s, a);
     }
     COME_CHECK_LAUNCH("come_attn_varlen_fwd");
+    if (plan.splits > 1) {
+        const dim3 cgrid(static_cast<unsigned>(n_seq * n_heads * plan.nb_tail));
+        if (dtype == COME_BF16) hipLaunchKernelGGL(attn_combine_kernel<COME_BF16>, cgrid, dim3(256), 0, s, a, kBlockM);
+        else hipLaunchKernelGGL(attn_combine_kernel<COME_F16>, cgrid, dim3(256), 0, s, a, kBlockM);
+        COME_CHECK_LAUNCH("come_attn_varlen_fwd (combine)");
+    }
     return COME_OK;
+}
+
+extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v, int dtype, int64_t q_row_stride,
+                                    int64_t q_head_stride, int64_t k_row_stride, int64_t k_head_stride,
+                                    int64_t v_row_stride, int64_t v_head_stride, const int32_t *cu_seqlens,
+                                    int64_t n_seq, int64_t total, int64_t n_heads, int64_t head_dim,
+                                    const void *perkey_bias, int64_t max_seqlen, float softmax_scale, void *out,
+                                    int64_t o_row_stride, int64_t o_head_stride, float *lse, void *stream) {
+    return come_attn_varlen_fwd_ws(q, k, v, dtype, q_row_stride, q_head_stride, k_row_stride, k_head_stride,
+                                   v_row_stride, v_head_stride, cu_seqlens, n_seq, total, n_heads, head_dim,
+                                   perkey_bias, max_seqlen, softmax_scale, out, o_row_stride, o_head_stride, lse,
+                                   nullptr, 0, stream);
 }

@@ -106,12 +106,16 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
             softmax_lse.fill_(-math.inf)
         if max_seqlen_k > 0:
             lib = _lib.load()
-            _lib.check(lib.come_attn_varlen_fwd(
+            # work buffer for the key-split tail of long launches (0 bytes: the launch does not use one)
+            work_bytes = lib.come_attn_work_bytes(batch_size, total_q, num_heads, max_seqlen_k)
+            work = torch.empty(work_bytes, dtype=torch.uint8, device=dev) if work_bytes > 0 else None
+            _lib.check(lib.come_attn_varlen_fwd_ws(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.dtype_code(q.dtype),
                 q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
                 cu_seqlens_q.data_ptr(), batch_size, total_q, num_heads, head_size,
                 _lib.ptr(perkey_bias), max_seqlen_k, float(softmax_scale),
-                out.data_ptr(), out.stride(0), out.stride(1), softmax_lse.data_ptr(), _lib.current_stream(dev)))
+                out.data_ptr(), out.stride(0), out.stride(1), softmax_lse.data_ptr(),
+                _lib.ptr(work), work_bytes, _lib.current_stream(dev)))
         else:
             out.zero_()
             softmax_lse.fill_(math.inf)

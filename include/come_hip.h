@@ -175,6 +175,30 @@ int come_attn_varlen_fwd(const void *q, const void *k, const void *v, int dtype,
                          float *lse, void *stream);
 
 /*
+ * come_attn_varlen_fwd_ws — the same operator with a caller-supplied work buffer.  When the launch would end
+ * in a partly filled last round of workgroups (long segments), the query blocks of that round are computed as
+ * several workgroups each, every one over its share of the keys, into `work`, and combined by a second small
+ * kernel: the result is the same up to rounding, the tail of the launch is shorter.
+ *
+ *   work, work_bytes   device buffer, 16-byte aligned, of at least come_attn_work_bytes(...) bytes; NULL or a
+ *                      smaller buffer makes the call identical to come_attn_varlen_fwd
+ * come_attn_work_bytes returns 0 when a launch of that shape would not use a buffer.
+ *
+ * No counterpart in the reference (its kernel has a split-KV variant for decoding only,
+ * src/cuda_extension/flash_attn/src/flash_fwd_launch_template.h:99-157, unreachable from the varlen forward).
+ */
+int64_t come_attn_work_bytes(int64_t n_seq, int64_t total, int64_t n_heads, int64_t max_seqlen);
+int come_attn_varlen_fwd_ws(const void *q, const void *k, const void *v, int dtype,
+                            int64_t q_row_stride, int64_t q_head_stride,
+                            int64_t k_row_stride, int64_t k_head_stride,
+                            int64_t v_row_stride, int64_t v_head_stride,
+                            const int32_t *cu_seqlens, int64_t n_seq, int64_t total,
+                            int64_t n_heads, int64_t head_dim,
+                            const void *perkey_bias, int64_t max_seqlen, float softmax_scale,
+                            void *out, int64_t o_row_stride, int64_t o_head_stride,
+                            float *lse, void *work, int64_t work_bytes, void *stream);
+
+/*
  * come_qk_norm_rope — attention prologue, in place on the packed projection output:
  * LayerNorm over the head dimension of every q and k head, then the 2-D rotary position
  * embedding.
