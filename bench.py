@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "copy", "e2e", "stress", "frame"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "copy", "e2e", "stress", "frame"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -249,6 +249,39 @@ def bench_merge_unmerge(device, iters=200, warmup=20):
                                  "unit": "GB/s", "frac": round(split_gbs / PEAK_HBM_GBS, 4),
                                  "traffic": TRAFFIC_BYTES["unmerge"]}},
     }
+
+
+def bench_unmerge_pair(device, w, iters=200, warmup=20):
+    """Retained-layer step of the fused aggregator: two packed tensors restored to the dense grid side by side
+    (``come_token_split_pair``), next to two ``come_token_split`` launches followed by ``torch.cat``."""
+    import torch
+    from come_amd import _lib
+
+    lib, stream = _lib.load(), _lib.current_stream(device)
+    rows, C, P, sets = w["frames"] * w["N"], w["C"], w["P"], len(w["outs"])
+    wide = [torch.empty(rows, 2 * C, dtype=torch.bfloat16, device=device) for _ in range(4)]
+    state = {"i": 0}
+
+    def pair():
+        i = state["i"] = (state["i"] + 1) % sets
+        _lib.check(lib.come_token_split_pair(w["outs"][i].data_ptr(), w["outs"][(i + 1) % sets].data_ptr(),
+                                             _lib.COME_BF16, P, C, None, w["index_map"].data_ptr(), rows,
+                                             wide[i % 4].data_ptr(), stream))
+
+    def two_and_cat():
+        i = state["i"] = (state["i"] + 1) % sets
+        for j in (i, (i + 1) % sets):
+            _lib.check(lib.come_token_split(w["outs"][j].data_ptr(), _lib.COME_BF16, P, C, None,
+                                            w["index_map"].data_ptr(), rows, w["restored"][j].data_ptr(), stream))
+        torch.cat((w["restored"][i], w["restored"][(i + 1) % sets]), dim=-1, out=wide[i % 4])
+
+    _, pair_ms = time_loop(pair, iters, warmup)
+    _, cat_ms = time_loop(two_and_cat, iters, warmup)
+    nbytes = 2 * P * C * 2 + rows * 4 + rows * 2 * C * 2
+    gbs = nbytes / (pair_ms / iters * 1e-3) / 1e9
+    return {"workload": "two packed [%d, %d] bf16 -> dense [%d, %d]" % (P, C, rows, 2 * C),
+            "us_per_call": round(pair_ms / iters * 1e3, 2), "algorithmic_bytes": nbytes, "GBs": round(gbs, 1),
+            "frac": round(gbs / PEAK_HBM_GBS, 4), "two_splits_and_cat_us": round(cat_ms / iters * 1e3, 2)}
 
 
 def bench_merge_ratios(device, iters=200, warmup=20):
@@ -491,6 +524,11 @@ def main():
             w, wall, ev_ms = bench_attention(args.steps, args.warmup, device)
             print(json.dumps({"only": "attn", "ms_per_call": ev_ms / args.steps,
                               "tflops": w["flops"] / (ev_ms / args.steps * 1e-3) / 1e12}))
+        elif args.only == "pair":
+            mw = merge_workload(device)
+            for _ in range(8):
+                mw["merge_only"]()
+            print(json.dumps({"only": "pair", **bench_unmerge_pair(device, mw, args.steps, args.warmup)}))
         else:
             mw = merge_workload(device)
             for _ in range(8):
@@ -532,6 +570,7 @@ def main():
     if not args.no_other:
         mw, other = bench_merge_unmerge(device)
         result["other"] = other
+        other["unmerge_pair"] = bench_unmerge_pair(device, mw)
         other["library_gemm_reference"] = bench_gemm_reference(device)
         other["merge_other_ratios"] = bench_merge_ratios(device)
         other["frame_attention"] = bench_frame_attention(device, w)

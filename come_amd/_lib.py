@@ -33,6 +33,7 @@ SIGNATURES = {
     "come_token_merge": (_int, [_ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                 _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "come_token_split": (_int, [_ptr, _int, _i64, _i64, _ptr, _ptr, _i64, _ptr, _ptr]),
+    "come_token_split_pair": (_int, [_ptr, _ptr, _int, _i64, _i64, _ptr, _ptr, _i64, _ptr, _ptr]),
     "come_select_windows": (_int, [_ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int, _f32,
                                    _ptr, _ptr, _ptr, _i64, _ptr]),
     "come_select_work_bytes": (_i64, [_i64, _i64, _i64, _i64, _i64, _i64]),

@@ -339,11 +339,14 @@ __global__ __launch_bounds__(kThreads) void merge_elem_kernel(const MergeArgs a)
 // ---------------------------------------------------------------------------------
 constexpr int kSplitRows = 1;      // output rows per thread (measured best of 1, 2, 3, 4, 8)
 
-template <typename IndexT>
-__global__ __launch_bounds__(kThreads) void split_vec_kernel(const uint4 *__restrict__ merged, int64_t merged_rows,
+// PAIR: two packed sources with one index map; an output row holds the row of `merged` followed by the row of
+// `merged_b` (`chunks` is the width of one source row, an output row has 2 * chunks chunks).
+template <typename IndexT, bool PAIR>
+__global__ __launch_bounds__(kThreads) void split_vec_kernel(const uint4 *__restrict__ merged,
+                                                             const uint4 *__restrict__ merged_b, int64_t merged_rows,
                                                              const IndexT *__restrict__ rev, int64_t total,
                                                              int chunks, uint4 *__restrict__ out, int64_t items,
-                                                             FastDiv by_chunks) {
+                                                             FastDiv by_out_chunks) {
     // workgroup i runs on XCD i % 8; dealing the output rows to the XCDs in runs of 256 keeps the (up to nine)
     // consumers of a merged row on one L2
     uint32_t bid = blockIdx.x;
@@ -354,8 +357,12 @@ __global__ __launch_bounds__(kThreads) void split_vec_kernel(const uint4 *__rest
     }
     const uint32_t id = bid * kThreads + threadIdx.x;               // items < 2^31 (checked by the host)
     if (id >= items) return;
-    const uint32_t quad = fast_div(id, by_chunks);
-    const int chunk = static_cast<int>(id - quad * chunks);
+    const int out_chunks = PAIR ? 2 * chunks : chunks;
+    const uint32_t quad = fast_div(id, by_out_chunks);
+    const int out_chunk = static_cast<int>(id - quad * out_chunks);
+    const bool second = PAIR && out_chunk >= chunks;
+    const uint4 *__restrict__ src = second ? merged_b : merged;
+    const int chunk = second ? out_chunk - chunks : out_chunk;
     const int64_t i0 = static_cast<int64_t>(quad) * kSplitRows;
     uint4 v[kSplitRows];
 #pragma unroll
@@ -363,32 +370,37 @@ __global__ __launch_bounds__(kThreads) void split_vec_kernel(const uint4 *__rest
         v[r] = make_uint4(0, 0, 0, 0);
         if (i0 + r < total) {
             const int64_t s = static_cast<int64_t>(rev[i0 + r]);
-            if (s >= 0 && s < merged_rows) v[r] = merged[s * chunks + chunk];
+            if (s >= 0 && s < merged_rows) v[r] = src[s * chunks + chunk];
         }
     }
 #pragma unroll
     for (int r = 0; r < kSplitRows; ++r)
-        if (i0 + r < total) st16_stream(out + (i0 + r) * chunks + chunk, v[r]);
+        if (i0 + r < total) st16_stream(out + (i0 + r) * out_chunks + out_chunk, v[r]);
 }
 
+// element-wise fallback; `pair`: output rows are [row of merged | row of merged_b]
 template <typename IndexT>
-__global__ __launch_bounds__(kThreads) void split_elem_kernel(const uint8_t *__restrict__ merged, int64_t merged_rows,
-                                                              const IndexT *__restrict__ rev, int64_t total,
-                                                              int64_t row_bytes, int elem_bytes,
+__global__ __launch_bounds__(kThreads) void split_elem_kernel(const uint8_t *__restrict__ merged,
+                                                              const uint8_t *__restrict__ merged_b, bool pair,
+                                                              int64_t merged_rows, const IndexT *__restrict__ rev,
+                                                              int64_t total, int64_t row_bytes, int elem_bytes,
                                                               uint8_t *__restrict__ out) {
     const int64_t id = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
     const int64_t per_row = row_bytes / elem_bytes;
-    if (id >= total * per_row) return;
-    const int64_t i = id / per_row;
-    const int64_t c = id - i * per_row;
+    const int64_t per_out = pair ? 2 * per_row : per_row;
+    if (id >= total * per_out) return;
+    const int64_t i = id / per_out;
+    const int64_t oc = id - i * per_out;
+    const bool second = oc >= per_row;
+    const uint8_t *__restrict__ src = second ? merged_b : merged;
+    const int64_t c = second ? oc - per_row : oc;
     const int64_t s = static_cast<int64_t>(rev[i]);
     const bool ok = s >= 0 && s < merged_rows;
     if (elem_bytes == 4) {
-        reinterpret_cast<uint32_t *>(out)[i * per_row + c] =
-            ok ? reinterpret_cast<const uint32_t *>(merged)[s * per_row + c] : 0u;
+        reinterpret_cast<uint32_t *>(out)[id] = ok ? reinterpret_cast<const uint32_t *>(src)[s * per_row + c] : 0u;
     } else {
-        reinterpret_cast<uint16_t *>(out)[i * per_row + c] =
-            ok ? reinterpret_cast<const uint16_t *>(merged)[s * per_row + c] : uint16_t(0);
+        reinterpret_cast<uint16_t *>(out)[id] =
+            ok ? reinterpret_cast<const uint16_t *>(src)[s * per_row + c] : uint16_t(0);
     }
 }
 
@@ -524,46 +536,68 @@ extern "C" int come_token_merge(const void *tokens, int dtype, int64_t rows, int
     return COME_OK;
 }
 
+// shared body of come_token_split (pair = false, merged_b unused) and come_token_split_pair
+static int token_split_impl(const char *who, bool pair, const void *merged, const void *merged_b, int dtype,
+                            int64_t merged_rows, int64_t chans, const int64_t *rev_i64, const int32_t *rev_i32,
+                            int64_t total, void *out, void *stream) {
+    COME_REQUIRE(dtype_ok(dtype), COME_ERR_UNSUPPORTED, "%s: unsupported dtype %d", who, dtype);
+    COME_REQUIRE(merged_rows >= 0 && chans >= 1 && total >= 0, COME_ERR_INVALID,
+                 "%s: negative size or chans < 1", who);
+    COME_REQUIRE((rev_i64 != nullptr) != (rev_i32 != nullptr) || total == 0, COME_ERR_INVALID,
+                 "%s: exactly one of rev_i64 / rev_i32 must be given", who);
+    if (total == 0) return COME_OK;
+    COME_REQUIRE(out != nullptr && (merged_rows == 0 || (merged != nullptr && (!pair || merged_b != nullptr))),
+                 COME_ERR_INVALID, "%s: merged / out is NULL", who);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t row_bytes = chans * dtype_bytes(dtype);
+    const bool vec = (row_bytes % 16 == 0) && aligned16(merged) && aligned16(merged_b) && aligned16(out);
+    if (vec) {
+        const int chunks = static_cast<int>(row_bytes / 16);
+        const int out_chunks = pair ? 2 * chunks : chunks;
+        const int64_t items = ceil_div(total, kSplitRows) * out_chunks;
+        const int64_t blocks = ceil_div(items, kThreads);
+        COME_REQUIRE(items < (1ll << 31), COME_ERR_UNSUPPORTED, "%s: problem too large for one launch", who);
+        const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+        const FastDiv by_out_chunks = make_fastdiv(out_chunks);
+        const uint4 *a4 = static_cast<const uint4 *>(merged), *b4 = static_cast<const uint4 *>(merged_b);
+        uint4 *o4 = static_cast<uint4 *>(out);
+#define COME_SPLIT_CASE(IDX_, PAIR_, REV_)                                                                       \
+    hipLaunchKernelGGL((split_vec_kernel<IDX_, PAIR_>), grid, block, 0, s, a4, b4, merged_rows, REV_, total,     \
+                       chunks, o4, items, by_out_chunks)
+        if (rev_i64 && pair) COME_SPLIT_CASE(int64_t, true, rev_i64);
+        else if (rev_i64) COME_SPLIT_CASE(int64_t, false, rev_i64);
+        else if (pair) COME_SPLIT_CASE(int32_t, true, rev_i32);
+        else COME_SPLIT_CASE(int32_t, false, rev_i32);
+#undef COME_SPLIT_CASE
+    } else {
+        const int eb = dtype_bytes(dtype);
+        const int64_t blocks = ceil_div(total * chans * (pair ? 2 : 1), kThreads);
+        COME_REQUIRE(blocks < (1ll << 31), COME_ERR_UNSUPPORTED, "%s: problem too large for one launch", who);
+        const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+        const uint8_t *a1 = static_cast<const uint8_t *>(merged), *b1 = static_cast<const uint8_t *>(merged_b);
+        if (rev_i64)
+            hipLaunchKernelGGL(split_elem_kernel<int64_t>, grid, block, 0, s, a1, b1, pair, merged_rows, rev_i64, total,
+                               row_bytes, eb, static_cast<uint8_t *>(out));
+        else
+            hipLaunchKernelGGL(split_elem_kernel<int32_t>, grid, block, 0, s, a1, b1, pair, merged_rows, rev_i32, total,
+                               row_bytes, eb, static_cast<uint8_t *>(out));
+    }
+    COME_CHECK_LAUNCH(who);
+    return COME_OK;
+}
+
 extern "C" int come_token_split(const void *merged, int dtype, int64_t merged_rows, int64_t chans,
                                 const int64_t *rev_i64, const int32_t *rev_i32, int64_t total, void *out,
                                 void *stream) {
     clear_error();
-    COME_REQUIRE(dtype_ok(dtype), COME_ERR_UNSUPPORTED, "come_token_split: unsupported dtype %d", dtype);
-    COME_REQUIRE(merged_rows >= 0 && chans >= 1 && total >= 0, COME_ERR_INVALID,
-                 "come_token_split: negative size or chans < 1");
-    COME_REQUIRE((rev_i64 != nullptr) != (rev_i32 != nullptr) || total == 0, COME_ERR_INVALID,
-                 "come_token_split: exactly one of rev_i64 / rev_i32 must be given");
-    if (total == 0) return COME_OK;
-    COME_REQUIRE(out != nullptr && (merged != nullptr || merged_rows == 0), COME_ERR_INVALID,
-                 "come_token_split: merged / out is NULL");
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const int64_t row_bytes = chans * dtype_bytes(dtype);
-    const bool vec = (row_bytes % 16 == 0) && aligned16(merged) && aligned16(out);
-    if (vec) {
-        const int chunks = static_cast<int>(row_bytes / 16);
-        const int64_t items = ceil_div(total, kSplitRows) * chunks;
-        const int64_t blocks = ceil_div(items, kThreads);
-        COME_REQUIRE(items < (1ll << 31), COME_ERR_UNSUPPORTED, "come_token_split: problem too large for one launch");
-        const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
-        const FastDiv by_chunks = make_fastdiv(chunks);
-        if (rev_i64)
-            hipLaunchKernelGGL(split_vec_kernel<int64_t>, grid, block, 0, s, static_cast<const uint4 *>(merged),
-                               merged_rows, rev_i64, total, chunks, static_cast<uint4 *>(out), items, by_chunks);
-        else
-            hipLaunchKernelGGL(split_vec_kernel<int32_t>, grid, block, 0, s, static_cast<const uint4 *>(merged),
-                               merged_rows, rev_i32, total, chunks, static_cast<uint4 *>(out), items, by_chunks);
-    } else {
-        const int eb = dtype_bytes(dtype);
-        const int64_t blocks = ceil_div(total * chans, kThreads);
-        COME_REQUIRE(blocks < (1ll << 31), COME_ERR_UNSUPPORTED, "come_token_split: problem too large for one launch");
-        const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
-        if (rev_i64)
-            hipLaunchKernelGGL(split_elem_kernel<int64_t>, grid, block, 0, s, static_cast<const uint8_t *>(merged),
-                               merged_rows, rev_i64, total, row_bytes, eb, static_cast<uint8_t *>(out));
-        else
-            hipLaunchKernelGGL(split_elem_kernel<int32_t>, grid, block, 0, s, static_cast<const uint8_t *>(merged),
-                               merged_rows, rev_i32, total, row_bytes, eb, static_cast<uint8_t *>(out));
-    }
-    COME_CHECK_LAUNCH("come_token_split");
-    return COME_OK;
+    return token_split_impl("come_token_split", false, merged, nullptr, dtype, merged_rows, chans, rev_i64, rev_i32, total,
+                            out, stream);
+}
+
+extern "C" int come_token_split_pair(const void *merged_a, const void *merged_b, int dtype, int64_t merged_rows,
+                                     int64_t chans, const int64_t *rev_i64, const int32_t *rev_i32, int64_t total,
+                                     void *out, void *stream) {
+    clear_error();
+    return token_split_impl("come_token_split_pair", true, merged_a, merged_b, dtype, merged_rows, chans, rev_i64, rev_i32,
+                            total, out, stream);
 }

@@ -20,6 +20,7 @@ from ... import _lib
 __all__ = [
     "co_me_token_merge_cuda",
     "co_me_token_split_cuda",
+    "co_me_token_split_pair_cuda",
     "co_me_token_merge_2d_cuda",
     "co_me_select_windows",
     "co_me_select_merge_2d",
@@ -96,6 +97,32 @@ def co_me_token_split_cuda(merged_flat: torch.Tensor, rev_id: torch.Tensor, C: i
         r32 = rev_c.data_ptr() if rev_c.dtype == torch.int32 else None
         _lib.check(lib.come_token_split(merged_c.data_ptr(), _lib.dtype_code(merged_c.dtype), merged_c.shape[0], C,
                                         r64, r32, total, out.data_ptr(), _lib.current_stream(dev)))
+    return out
+
+
+def co_me_token_split_pair_cuda(merged_a: torch.Tensor, merged_b: torch.Tensor, rev_id: torch.Tensor,
+                                C: int) -> torch.Tensor:
+    """Two token splits and the concatenation of their results in one launch:
+    ``out[i] = cat(merged_a[rev_id[i]], merged_b[rev_id[i]])`` -> ``[total, 2 * C]``
+    (the retained-layer step of the fused aggregator, reference ``vggt/fused.py:157-165``)."""
+    _torch_check(merged_a.is_cuda and merged_b.is_cuda, "merged_a and merged_b must be on CUDA")
+    _torch_check(rev_id.is_cuda, "rev_id must be on CUDA")
+    _torch_check(merged_a.dim() == 2 and merged_a.shape[1] == C, "merged_a must be [P, C]")
+    _torch_check(merged_b.shape == merged_a.shape and merged_b.dtype == merged_a.dtype
+                 and merged_b.device == merged_a.device, "merged_b must match merged_a in shape, dtype and device")
+    _torch_check(rev_id.dtype in (torch.int64, torch.int32), "rev_id must be int64 or int32")
+    lib = _lib.load()
+    a_c, b_c = merged_a.contiguous(), merged_b.contiguous()
+    rev_c = rev_id.contiguous().reshape(-1)
+    total = rev_c.shape[0]
+    dev = a_c.device
+    with torch.cuda.device(dev):
+        out = torch.empty(total, 2 * C, dtype=a_c.dtype, device=dev)
+        r64 = rev_c.data_ptr() if rev_c.dtype == torch.int64 else None
+        r32 = rev_c.data_ptr() if rev_c.dtype == torch.int32 else None
+        _lib.check(lib.come_token_split_pair(a_c.data_ptr(), b_c.data_ptr(), _lib.dtype_code(a_c.dtype),
+                                             a_c.shape[0], C, r64, r32, total, out.data_ptr(),
+                                             _lib.current_stream(dev)))
     return out
 
 

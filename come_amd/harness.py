@@ -204,10 +204,14 @@ class AlternatingAggregator(nn.Module):
             state["x"] = x_glob
             if i in cfg.taps:
                 if state["ctx"] is not None:
-                    def restore(t):
-                        jag = JaggedTokens(tokens=t.unsqueeze(0), weight=state["weight"], offset=state["offset"])
-                        return merger.split(state["ctx"], state["stub"], jag).reshape(B * S * N, C)
-                    taps.append(torch.cat((restore(x_frame), restore(x_glob)), dim=-1))
+                    def jagged(t):
+                        return JaggedTokens(tokens=t.unsqueeze(0), weight=state["weight"], offset=state["offset"])
+                    if hasattr(merger, "split_pair"):      # both splits and the concatenation in one launch
+                        tap = merger.split_pair(state["ctx"], state["stub"], jagged(x_frame), jagged(x_glob))
+                        taps.append(tap.reshape(B * S * N, 2 * C))
+                    else:
+                        taps.append(torch.cat([merger.split(state["ctx"], state["stub"], jagged(t))
+                                               .reshape(B * S * N, C) for t in (x_frame, x_glob)], dim=-1))
                 else:
                     taps.append(torch.cat((x_frame, x_glob), dim=-1))
         info["maps"] = self.dense_head(taps, B, S, gh, gw)

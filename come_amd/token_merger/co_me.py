@@ -55,6 +55,15 @@ def func_token_split(tokens: JaggedTokens, rev_id: torch.Tensor,
     return restored.reshape(B * S, N, C)
 
 
+def func_token_split_pair(tokens_a: JaggedTokens, tokens_b: JaggedTokens, rev_id: torch.Tensor,
+                          bsnc_shape: tuple[int, int, int, int]) -> torch.Tensor:
+    """``torch.cat((func_token_split(a), func_token_split(b)), dim=-1)`` in one launch -> ``[B*S, N, 2*C]``."""
+    B, S, N, C = bsnc_shape
+    restored = co_me_cuext.co_me_token_split_pair_cuda(tokens_a.tokens.squeeze(0), tokens_b.tokens.squeeze(0),
+                                                       rev_id.contiguous(), C)
+    return restored.reshape(B * S, N, 2 * C)
+
+
 class CoMe_TokenMerger(ITokenMerger):
     """Groups of ``group_size`` consecutive tokens (reference ``CoMe_TokenMerger``, co_me.py:20-105).
 
@@ -98,6 +107,12 @@ class CoMe_TokenMerger(ITokenMerger):
         rev_id, shape_bsnc = stub
         B, S, N, C = shape_bsnc
         return func_token_split(tokens, rev_id, shape_bsnc).view(B, S, N, C)
+
+    def split_pair(self, ctx, stub: Any, tokens_a: JaggedTokens, tokens_b: JaggedTokens) -> torch.Tensor:
+        """``torch.cat((split(a), split(b)), dim=-1)`` in one launch -> ``[B, S, N, 2*C]``."""
+        rev_id, shape_bsnc = stub
+        B, S, N, C = shape_bsnc
+        return func_token_split_pair(tokens_a, tokens_b, rev_id, shape_bsnc).view(B, S, N, 2 * C)
 
     def build_infer_mask(self, ctx) -> torch.Tensor:
         mask, (B, S, _, H, W) = ctx

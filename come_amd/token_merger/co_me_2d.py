@@ -21,7 +21,7 @@ import torch
 
 from ..cuda_extension.co_me import co_me_cuext
 from ..interface import ITokenMerger, JaggedTokens
-from .co_me import func_token_split
+from .co_me import func_token_split, func_token_split_pair
 
 
 def _validate_token_merge_2d_args(tokens, start_index, group_h, group_w, H, W, merge_mask,
@@ -108,6 +108,12 @@ class CoMe_2D_TokenMerger(ITokenMerger):
         rev_id, shape_bsnc = stub
         B, S, N, C = shape_bsnc
         return func_token_split(tokens, rev_id, shape_bsnc).view(B, S, N, C)
+
+    def split_pair(self, ctx: Any, stub: Any, tokens_a: JaggedTokens, tokens_b: JaggedTokens) -> torch.Tensor:
+        """``torch.cat((split(a), split(b)), dim=-1)`` in one launch -> ``[B, S, N, 2*C]``."""
+        rev_id, shape_bsnc = stub
+        B, S, N, C = shape_bsnc
+        return func_token_split_pair(tokens_a, tokens_b, rev_id, shape_bsnc).view(B, S, N, 2 * C)
 
     def build_infer_mask(self, ctx: Any) -> torch.Tensor:
         """``[B, S, H, W] bool``: True where the patch was merged (positions outside full windows: False)."""

@@ -114,6 +114,24 @@ int come_token_split(const void *merged, int dtype, int64_t merged_rows, int64_t
                      void *out, void *stream);
 
 /*
+ * come_token_split_pair — unmerge two packed tensors that share one index map into one
+ * dense tensor with their channels side by side:
+ *   out[i, :chans] = merged_a[rev[i], :],  out[i, chans:] = merged_b[rev[i], :].
+ *
+ *   merged_a, merged_b  [merged_rows, chans] of `dtype`, contiguous
+ *   out                 [total, 2 * chans] of `dtype`
+ * Other arguments and the out-of-range rule as for come_token_split.
+ *
+ * Stands in for the two token splits followed by torch.cat(dim=-1) at the retained layers
+ * of the fused aggregator (src/accelerate/vggt/fused.py:157-165): one launch and one pass
+ * over the output instead of two splits plus a concatenation.
+ */
+int come_token_split_pair(const void *merged_a, const void *merged_b, int dtype,
+                          int64_t merged_rows, int64_t chans,
+                          const int64_t *rev_i64, const int32_t *rev_i32, int64_t total,
+                          void *out, void *stream);
+
+/*
  * come_select_windows — per-window confidence mean and lowest-confidence selection.
  *
  *   conf     [batch * frames, grid_h, grid_w] of `dtype` (COME_BF16 or COME_F32), contiguous

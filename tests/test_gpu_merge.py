@@ -170,3 +170,57 @@ def test_full_size_c2_properties():
     assert torch.equal(rev2, rev)
     diff = (jag2.tokens.float() - jag.tokens.float()).abs()
     assert float(diff.max()) <= 1e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("C", [1024, 64, 12, 2, 1])
+@pytest.mark.parametrize("index_dtype", [torch.int64, torch.int32], ids=["i64", "i32"])
+def test_split_pair_is_two_splits_side_by_side(dtype, C, index_dtype):
+    # the retained-layer step of the fused aggregator (reference vggt/fused.py:157-165): two token splits + cat
+    P, total = 777, 2500
+    g = torch.Generator().manual_seed(C)
+    a = torch.randn(P, C, generator=g).to(dtype)
+    b = torch.randn(P, C, generator=g).to(dtype)
+    rev = torch.randint(0, P, (total,), generator=g)
+    want = torch.cat((a[rev], b[rev]), dim=-1)                                    # a gather is bit-exact
+    a_d, b_d, rev_d = a.to(DEV), b.to(DEV), rev.to(index_dtype).to(DEV)
+    got = co_me_cuext.co_me_token_split_pair_cuda(a_d, b_d, rev_d, C)
+    assert got.shape == (total, 2 * C) and got.dtype == dtype
+    assert torch.equal(got.cpu(), want)
+    assert torch.equal(got[:, :C], co_me_cuext.co_me_token_split_cuda(a_d, rev_d, C))
+    assert torch.equal(got[:, C:], co_me_cuext.co_me_token_split_cuda(b_d, rev_d, C))
+
+
+def test_split_pair_edges_and_errors():
+    C = 256
+    a = torch.randn(10, C).bfloat16().to(DEV)
+    b = torch.randn(10, C).bfloat16().to(DEV)
+    rev = torch.tensor([0, 9, -1, 10, 3], device=DEV)                              # out-of-range rows come back as zeros
+    got = co_me_cuext.co_me_token_split_pair_cuda(a, b, rev, C).cpu()
+    assert torch.equal(got[0], torch.cat((a[0], b[0])).cpu()) and torch.equal(got[4], torch.cat((a[3], b[3])).cpu())
+    assert float(got[2].abs().max()) == 0 and float(got[3].abs().max()) == 0
+    empty = co_me_cuext.co_me_token_split_pair_cuda(a, b, rev[:0], C)
+    assert empty.shape == (0, 2 * C)
+    no_rows = co_me_cuext.co_me_token_split_pair_cuda(a[:0], b[:0], rev, C)
+    assert no_rows.shape == (5, 2 * C) and float(no_rows.abs().max()) == 0
+    with pytest.raises(RuntimeError, match="merged_b must match"):
+        co_me_cuext.co_me_token_split_pair_cuda(a, b[:5], rev, C)
+    with pytest.raises(RuntimeError, match="merged_b must match"):
+        co_me_cuext.co_me_token_split_pair_cuda(a, b.float(), rev, C)
+    with pytest.raises(RuntimeError, match="rev_id must be"):
+        co_me_cuext.co_me_token_split_pair_cuda(a, b, rev.float(), C)
+
+
+def test_split_pair_full_size_through_the_merger():
+    from come_amd.token_merger import func_token_split_pair
+    B, H, W, S, C = 16, 37, 37, 5, 1024
+    g = torch.Generator().manual_seed(1)
+    tokens = torch.randn(B, S + H * W, C, generator=g).bfloat16().to(DEV)
+    mask = (torch.rand(B, 144, generator=g) < 0.5).to(DEV)
+    jag, rev = func_token_merge_2d(tokens, S, 3, 3, H, W, mask, allow_remainder=True)
+    other = type(jag)(tokens=jag.tokens.flip(1).contiguous(), weight=jag.weight, offset=jag.offset)
+    shape = (1, B, S + H * W, C)
+    both = func_token_split_pair(jag, other, rev, shape)
+    assert both.shape == (B, S + H * W, 2 * C)
+    assert torch.equal(both[..., :C], func_token_split(jag, rev, shape))
+    assert torch.equal(both[..., C:], func_token_split(other, rev, shape))
