@@ -71,10 +71,6 @@ def _default_prologue(qkv, q_norm, k_norm, rope_base, pos, max_position):
 _ROPES: dict = {}
 
 
-def _max_seqlen(cu_seqlens: torch.Tensor) -> int:
-    return int((cu_seqlens[1:] - cu_seqlens[:-1]).max().item())
-
-
 class JaggedBlock(nn.Module):
     """Pre-norm transformer block on packed tokens ``[P, C]``."""
 
@@ -179,9 +175,12 @@ class AlternatingAggregator(nn.Module):
                      pos=pos.reshape(-1, 2).contiguous())
 
         def segments():
+            # the attention operator takes any upper bound of the segment lengths: the dense frame / sequence lengths
+            # are known without reading the merged offsets back (the reference reads the maximum in every layer,
+            # flash_attn/__init__.py:21-33)
             frame = state["offset"].to(torch.int32)
             glob = state["offset"][::S].to(torch.int32)
-            return (frame, _max_seqlen(frame)), (glob, _max_seqlen(glob))
+            return (frame, N), (glob, S * N)
 
         (cu_f, max_f), (cu_g, max_g) = segments()
         taps: list[torch.Tensor] = []

@@ -80,3 +80,22 @@ def test_work_buffer_rules():
                                            bias.data_ptr(), P, 0.125, out.data_ptr(), out.stride(0), out.stride(1), None,
                                            small.data_ptr(), small.numel(), _lib.current_stream(qkv.device)))
     assert torch.equal(out, ref_out)
+
+
+@pytest.mark.parametrize("lens", [[700, 300, 812], [9000, 700], [6000, 5000]], ids=str)
+def test_max_seqlen_may_be_any_upper_bound(lens):
+    """A caller that does not want to read the longest segment back from the device (the per-layer ``.item()`` of
+    reference flash_attn/__init__.py:21-33) passes a static bound such as the unmerged frame length or the total."""
+    P = sum(lens)
+    g = torch.Generator().manual_seed(P)
+    qkv = torch.randn(P, 3, H, D, generator=g).bfloat16().to(DEV)
+    bias = (torch.rand(P, generator=g) * 3).log().clamp(min=-4).bfloat16().to(DEV)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32).to(DEV)
+    exact, exact_lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, max(lens), perkey_bias=bias,
+                                                                        softmax_scale=0.125, return_attn_probs=True)
+    for bound in (max(lens) + 1, max(lens) + 700, P, 2 * P):
+        out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, bound, perkey_bias=bias,
+                                                                     softmax_scale=0.125, return_attn_probs=True)
+        # the launch plan (workgroup width, key-split tail) may differ with the bound: same products, other order
+        torch.testing.assert_close(out.float(), exact.float(), atol=4e-3, rtol=2 ** -7)
+        torch.testing.assert_close(lse, exact_lse, atol=2e-3, rtol=1e-4)
