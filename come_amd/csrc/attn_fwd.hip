@@ -112,6 +112,14 @@ __device__ inline s16x4 lds_read_tr(const uint16_t *p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(p));
 }
 
+// Offsets come from device memory that the host cannot check: a segment is clamped into [0, total], so that
+// inconsistent offsets give wrong results for their rows instead of accesses outside the tensors.
+__device__ inline void segment_of(const AttnArgs &a, int seq, int &seq_start, int &L) {
+    const int total = static_cast<int>(a.total);
+    seq_start = min(max(a.cu[seq], 0), total);
+    L = min(max(a.cu[seq + 1], seq_start), total) - seq_start;
+}
+
 // Which (segment, head, query block) a workgroup computes.  Workgroup i is dispatched to XCD
 // i % 8, each XCD with its own L2: the query blocks of one (segment, head) unit run back to back
 // on one XCD and share that unit's K/V there, and units are dealt to the XCDs round-robin so that
@@ -214,8 +222,8 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
 
     int mblk, head, seq, tail, ks;
     if (!locate_block(a, mblk, head, seq, tail, ks)) return;
-    const int seq_start = a.cu[seq];
-    const int L = a.cu[seq + 1] - seq_start;
+    int seq_start, L;
+    segment_of(a, seq, seq_start, L);
     const int n_qblocks = (L + kBlockM - 1) / kBlockM;
     if (tail >= 0) {
         mblk = n_qblocks - a.nb_tail + tail;          // split workgroup: one of the unit's last query blocks
@@ -704,8 +712,8 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const AttnArgs a, int
     const int unit = blockIdx.x / a.nb_tail;
     const int head = unit % a.n_heads;
     const int seq = unit / a.n_heads;
-    const int seq_start = a.cu[seq];
-    const int L = a.cu[seq + 1] - seq_start;
+    int seq_start, L;
+    segment_of(a, seq, seq_start, L);
     const int mblk = (L + block_m - 1) / block_m - a.nb_tail + tail;
     if (mblk < 0) return;
     const int q0 = mblk * block_m;

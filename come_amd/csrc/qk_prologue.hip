@@ -38,10 +38,24 @@ __device__ inline void round_to_dtype(float *f) {
     Vec16<DT>::unpack(r, f);
 }
 
+// Lane exchanges inside a group of eight lanes as data-parallel-primitive moves (no LDS traffic, no address
+// arithmetic).  kSwapPairs / kSwapQuadHalves permute inside a quad of lanes (lane ^ 1, lane ^ 2);
+// kMirrorEight reverses the eight lanes of a half row (lane i <-> 7 - i).
+constexpr int kSwapPairs = 0xB1;           // quad_perm [1, 0, 3, 2]
+constexpr int kSwapQuadHalves = 0x4E;      // quad_perm [2, 3, 0, 1]
+constexpr int kMirrorEight = 0x141;        // row_half_mirror
+
+template <int CTRL>
+__device__ inline float lane_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+// Sum over the eight lanes of a head, the same in every lane: after the two steps inside the quads each quad
+// holds its sum in all four lanes, and the mirrored lane then belongs to the other quad.
 __device__ inline float group8_sum(float v) {
-    v += __shfl_xor(v, 1);
-    v += __shfl_xor(v, 2);
-    v += __shfl_xor(v, 4);
+    v += lane_move<kSwapPairs>(v);
+    v += lane_move<kSwapQuadHalves>(v);
+    v += lane_move<kMirrorEight>(v);
     return v;
 }
 
@@ -120,14 +134,15 @@ __global__ void __launch_bounds__(256) qk_norm_rope_kernel(const QkArgs a) {
             const float sign = (lane8 & 2) ? 1.f : -1.f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float partner = __shfl_xor(f[i], 2);
-                r[i] = sign * partner * sn[i];
+                r[i] = lane_move<kSwapQuadHalves>(f[i]) * sn[i];
                 f[i] = f[i] * c[i];
             }
             round_to_dtype<DT>(r);
             round_to_dtype<DT>(f);
+            // the rotated partner enters with sign -1 in the first half of each 32-element block (rounding is
+            // symmetric, so the sign can wait until the sum)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) f[i] += r[i];
+            for (int i = 0; i < 8; ++i) f[i] = fmaf(sign, r[i], f[i]);
         }
         if (live[t]) *p[t] = V::pack(f);
     }
