@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "copy", "e2e", "stress", "frame"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "copy", "e2e", "stress", "stress_e2e", "frame"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -386,9 +386,10 @@ def bench_gemm_reference(device):
             "frac_of_nominal_peak": round(tflops / PEAK_BF16_TFLOPS, 4)}
 
 
-def bench_e2e(device, frames=32, depth=24, reps=5):
+def bench_e2e(device, frames=32, depth=24, reps=5, height=518, width=518, ratio=0.5):
     """End-to-end aggregator (random init, bf16): 24 frame + 24 global blocks, dim 1024, 16 heads x 64, MLP 4096,
-    32 frames of 518x518; 3x3 merge from block 4 onward at ratio 0.5 against the same model without merging."""
+    32 frames of 518x518; 3x3 merge from block 4 onward at ratio 0.5 against the same model without merging.
+    (``frames=128, width=392, ratio=0.75``: the long-sequence stress shape, 133 248 tokens.)"""
     import torch
     from come_amd.harness import AggregatorConfig, AlternatingAggregator, relative_l1
     from come_amd.token_merger import CoMe_2D_TokenMerger
@@ -396,8 +397,9 @@ def bench_e2e(device, frames=32, depth=24, reps=5):
     torch.manual_seed(0)
     cfg = AggregatorConfig(depth=depth)
     model = AlternatingAggregator(cfg).eval().to(device=device, dtype=torch.bfloat16)
-    images = torch.rand(1, frames, 3, 518, 518, generator=torch.Generator().manual_seed(0)).to(device)
-    merger = CoMe_2D_TokenMerger(cfg.specials, 3, 3, 0.5, allow_remainder=True)
+    images = torch.rand(1, frames, 3, height, width, generator=torch.Generator().manual_seed(0)).to(device)
+    merger = CoMe_2D_TokenMerger(cfg.specials, 3, 3, ratio, allow_remainder=True)
+    gh, gw = height // 14, width // 14
 
     def timed(m):
         out = model(images, merger=m)                           # warm-up (allocator, GEMM heuristics)
@@ -412,13 +414,14 @@ def bench_e2e(device, frames=32, depth=24, reps=5):
 
     dense, dense_ms = timed(None)
     merged, merged_ms = timed(merger)
-    mask = merged["merge_mask"].reshape(frames, 12, 12)
-    keep = torch.ones(frames, 37, 37, dtype=torch.bool, device=device)
-    keep[:, :36, :36] = ~mask.repeat_interleave(3, 1).repeat_interleave(3, 2)
+    mh, mw = gh // 3, gw // 3
+    mask = merged["merge_mask"].reshape(frames, mh, mw)
+    keep = torch.ones(frames, gh, gw, dtype=torch.bool, device=device)
+    keep[:, :mh * 3, :mw * 3] = ~mask.repeat_interleave(3, 1).repeat_interleave(3, 2)
     keep_px = keep.repeat_interleave(14, 1).repeat_interleave(14, 2)[None, :, None]
     return {"workload": f"VGGT-style aggregator, random init, bf16: {depth} frame + {depth} global blocks, dim 1024, "
-                        f"16 heads x 64, MLP 4096, S={frames} frames 518x518 ({dense['tokens_dense']} tokens); 3x3 merge "
-                        f"from block {cfg.merge_block} at r=0.5 ({merged['tokens_packed']} packed tokens)",
+                        f"16 heads x 64, MLP 4096, S={frames} frames {height}x{width} ({dense['tokens_dense']} tokens); "
+                        f"3x3 merge from block {cfg.merge_block} at r={ratio} ({merged['tokens_packed']} packed tokens)",
             "merged_ms": round(merged_ms, 2), "unmerged_ms": round(dense_ms, 2),
             "speedup": round(dense_ms / merged_ms, 3), "reps": reps, "statistic": "median wall time per forward",
             "rel_l1_unmerged_windows": round(relative_l1(merged["maps"], dense["maps"], keep_px), 5),
@@ -511,6 +514,9 @@ def main():
             print(json.dumps({"only": "frame", **bench_frame_attention(device, None)}))
         elif args.only == "e2e":
             print(json.dumps({"only": "e2e", **bench_e2e(device, reps=max(1, args.steps))}))
+        elif args.only == "stress_e2e":                          # seconds per forward: not part of the default run
+            print(json.dumps({"only": "stress_e2e", **bench_e2e(device, frames=128, width=392, ratio=0.75,
+                                                                  reps=max(1, min(args.steps, 3)))}))
         elif args.only == "copy":
             # plain device copy of known size: the yardstick the HBM byte counters are scaled by
             nbytes = 256 << 20
