@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "copy", "e2e", "stress", "stress_e2e", "frame"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "copy", "e2e", "stress", "stress_e2e", "frame"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -164,19 +164,21 @@ def jittered_frame_masks(conf, ratio, jitter, seed):
     return rank < k[:, None]
 
 
-def merge_workload(device, ratio=0.5, sets=8, frames=16, H=37, W=37, jitter=None):
+def merge_workload(device, ratio=0.5, sets=8, frames=16, H=37, W=37, jitter=None, dtype=None, C=1024):
     """Merge microbenchmark: 16 frames, 37x37 patches + 5 specials, C = 1024, bf16.  ``sets`` rotating
     input / output buffer sets keep the working set (> 500 MB) out of the 256 MB Infinity Cache.  With ``jitter``
     the mask comes from ``jittered_frame_masks`` instead of the joint quantile selection."""
     import torch
     from come_amd import _lib
 
-    S0, C = 5, 1024
+    S0 = 5
     N = S0 + H * W
+    dtype = torch.bfloat16 if dtype is None else dtype
+    code, esize = _lib.dtype_code(dtype), torch.empty(0, dtype=dtype).element_size()
     lib = _lib.load()
     conf = smooth_confidence(frames, H, W, seed=0).to(device)
     torch.manual_seed(0)
-    tokens = [torch.randn(frames, N, C, device=device).bfloat16() for _ in range(sets)]
+    tokens = [torch.randn(frames, N, C, device=device).to(dtype) for _ in range(sets)]
     M = (H // 3) * (W // 3)
     tail = H * W - M * 9
     mask = torch.empty(frames, M, dtype=torch.uint8, device=device)
@@ -197,15 +199,15 @@ def merge_workload(device, ratio=0.5, sets=8, frames=16, H=37, W=37, jitter=None
 
     select_and_plan()
     P = int(offsets[-1].item())
-    outs = [torch.empty(P, C, dtype=torch.bfloat16, device=device) for _ in range(sets)]
+    outs = [torch.empty(P, C, dtype=dtype, device=device) for _ in range(sets)]
     index_map = torch.empty(frames * N, dtype=torch.int32, device=device)
     counts = torch.empty(P, dtype=torch.int32, device=device)
-    restored = [torch.empty(frames * N, C, dtype=torch.bfloat16, device=device) for _ in range(sets)]
+    restored = [torch.empty(frames * N, C, dtype=dtype, device=device) for _ in range(sets)]
     state = {"i": 0}
 
     def merge_only():
         i = state["i"] = (state["i"] + 1) % sets
-        _lib.check(lib.come_token_merge(tokens[i].data_ptr(), _lib.COME_BF16, frames, N, C, S0, 3, 3, H, W,
+        _lib.check(lib.come_token_merge(tokens[i].data_ptr(), code, frames, N, C, S0, 3, 3, H, W,
                                         mask.data_ptr(), offsets.data_ptr(), prefix.data_ptr(), outs[i].data_ptr(), P,
                                         None, index_map.data_ptr(), None, counts.data_ptr(), stream))
 
@@ -215,11 +217,12 @@ def merge_workload(device, ratio=0.5, sets=8, frames=16, H=37, W=37, jitter=None
 
     def split_only():
         i = state["i"] = (state["i"] + 1) % sets
-        _lib.check(lib.come_token_split(outs[i].data_ptr(), _lib.COME_BF16, P, C, None, index_map.data_ptr(),
+        _lib.check(lib.come_token_split(outs[i].data_ptr(), code, P, C, None, index_map.data_ptr(),
                                         frames * N, restored[i].data_ptr(), stream))
 
-    merge_bytes = frames * N * C * 2 + P * C * 2 + frames * N * 4 + P * 4 + frames * H * W * 4 + (frames + 1) * 4
-    split_bytes = P * C * 2 + frames * N * 4 + frames * N * C * 2
+    merge_bytes = (frames * N * C * esize + P * C * esize + frames * N * 4 + P * 4 + frames * H * W * 4
+                   + (frames + 1) * 4)
+    split_bytes = P * C * esize + frames * N * 4 + frames * N * C * esize
     return dict(merge_only=merge_only, pipeline=pipeline, split_only=split_only, P=P, merge_bytes=merge_bytes,
                 split_bytes=split_bytes, frames=frames, N=N, C=C, ratio=ratio, tokens=tokens, conf=conf,
                 counts=counts, offsets=offsets, outs=outs, restored=restored, index_map=index_map,
@@ -251,6 +254,27 @@ def bench_merge_unmerge(device, iters=200, warmup=20):
     }
 
 
+def bench_merge_caller_dtypes(device, iters=200, warmup=20):
+    """The two other tensors the fused aggregator of the reference merges (vggt/fused.py:126-129): the fp32 residual
+    stream [frames, N, 1024] and the bf16 positions [frames, N, 2] (element-wise kernels: rows of 4 bytes)."""
+    import torch
+
+    out = {}
+    for name, dtype, C in (("fp32_c1024", torch.float32, 1024), ("bf16_c2", torch.bfloat16, 2)):
+        w = merge_workload(device, dtype=dtype, C=C, sets=8 if C > 2 else 2)
+        for _ in range(8):
+            w["merge_only"]()
+        _, m_ms = time_loop(w["merge_only"], iters, warmup)
+        _, s_ms = time_loop(w["split_only"], iters, warmup)
+        out[name] = {"merge_us": round(m_ms / iters * 1e3, 2), "merge_bytes": w["merge_bytes"],
+                     "merge_GBs": round(w["merge_bytes"] / (m_ms / iters * 1e-3) / 1e9, 1),
+                     "unmerge_us": round(s_ms / iters * 1e3, 2), "unmerge_bytes": w["split_bytes"],
+                     "unmerge_GBs": round(w["split_bytes"] / (s_ms / iters * 1e-3) / 1e9, 1)}
+        del w
+        torch.cuda.empty_cache()
+    return out
+
+
 def bench_unmerge_pair(device, w, iters=200, warmup=20):
     """Retained-layer step of the fused aggregator: two packed tensors restored to the dense grid side by side
     (``come_token_split_pair``), next to two ``come_token_split`` launches followed by ``torch.cat``."""
@@ -259,21 +283,22 @@ def bench_unmerge_pair(device, w, iters=200, warmup=20):
 
     lib, stream = _lib.load(), _lib.current_stream(device)
     rows, C, P, sets = w["frames"] * w["N"], w["C"], w["P"], len(w["outs"])
-    wide = [torch.empty(rows, 2 * C, dtype=torch.bfloat16, device=device) for _ in range(4)]
+    wide = [torch.empty(rows, 2 * C, dtype=torch.bfloat16, device=device) for _ in range(sets)]
+    far = sets // 2                     # the second source was last touched half a rotation (> 256 MB of traffic) ago
     state = {"i": 0}
 
     def pair():
         i = state["i"] = (state["i"] + 1) % sets
-        _lib.check(lib.come_token_split_pair(w["outs"][i].data_ptr(), w["outs"][(i + 1) % sets].data_ptr(),
+        _lib.check(lib.come_token_split_pair(w["outs"][i].data_ptr(), w["outs"][(i + far) % sets].data_ptr(),
                                              _lib.COME_BF16, P, C, None, w["index_map"].data_ptr(), rows,
-                                             wide[i % 4].data_ptr(), stream))
+                                             wide[i].data_ptr(), stream))
 
     def two_and_cat():
         i = state["i"] = (state["i"] + 1) % sets
-        for j in (i, (i + 1) % sets):
+        for j in (i, (i + far) % sets):
             _lib.check(lib.come_token_split(w["outs"][j].data_ptr(), _lib.COME_BF16, P, C, None,
                                             w["index_map"].data_ptr(), rows, w["restored"][j].data_ptr(), stream))
-        torch.cat((w["restored"][i], w["restored"][(i + 1) % sets]), dim=-1, out=wide[i % 4])
+        torch.cat((w["restored"][i], w["restored"][(i + far) % sets]), dim=-1, out=wide[i])
 
     _, pair_ms = time_loop(pair, iters, warmup)
     _, cat_ms = time_loop(two_and_cat, iters, warmup)
@@ -530,6 +555,8 @@ def main():
             w, wall, ev_ms = bench_attention(args.steps, args.warmup, device)
             print(json.dumps({"only": "attn", "ms_per_call": ev_ms / args.steps,
                               "tflops": w["flops"] / (ev_ms / args.steps * 1e-3) / 1e12}))
+        elif args.only == "dtypes":
+            print(json.dumps({"only": "dtypes", **bench_merge_caller_dtypes(device, args.steps, args.warmup)}))
         elif args.only == "pair":
             mw = merge_workload(device)
             for _ in range(8):
@@ -579,6 +606,7 @@ def main():
         other["unmerge_pair"] = bench_unmerge_pair(device, mw)
         other["library_gemm_reference"] = bench_gemm_reference(device)
         other["merge_other_ratios"] = bench_merge_ratios(device)
+        other["merge_caller_dtypes"] = bench_merge_caller_dtypes(device)
         other["frame_attention"] = bench_frame_attention(device, w)
         other["stress"] = bench_stress(device)
     if not args.no_e2e:

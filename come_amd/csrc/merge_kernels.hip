@@ -338,6 +338,10 @@ __global__ __launch_bounds__(kThreads) void merge_elem_kernel(const MergeArgs a)
 // unmerge: out[i, :] = merged[rev[i], :]
 // ---------------------------------------------------------------------------------
 constexpr int kSplitRows = 1;      // output rows per thread (measured best of 1, 2, 3, 4, 8)
+#ifndef COME_SPLIT_RUN_ROWS
+#define COME_SPLIT_RUN_ROWS 256
+#endif
+constexpr int kSplitRunRows = COME_SPLIT_RUN_ROWS;   // output rows that stay on one XCD
 
 // PAIR: two packed sources with one index map; an output row holds the row of `merged` followed by the row of
 // `merged_b` (`chunks` is the width of one source row, an output row has 2 * chunks chunks).
@@ -346,14 +350,13 @@ __global__ __launch_bounds__(kThreads) void split_vec_kernel(const uint4 *__rest
                                                              const uint4 *__restrict__ merged_b, int64_t merged_rows,
                                                              const IndexT *__restrict__ rev, int64_t total,
                                                              int chunks, uint4 *__restrict__ out, int64_t items,
-                                                             FastDiv by_out_chunks) {
-    // workgroup i runs on XCD i % 8; dealing the output rows to the XCDs in runs of 256 keeps the (up to nine)
-    // consumers of a merged row on one L2
+                                                             FastDiv by_out_chunks, uint32_t run) {
+    // workgroup i runs on XCD i % 8; dealing the output rows to the XCDs in runs of `run` consecutive workgroups
+    // (kSplitRunRows output rows) keeps the (up to nine) consumers of a merged row on one L2
     uint32_t bid = blockIdx.x;
-    constexpr uint32_t kChunk = 128;                                 // consecutive workgroups (256 output rows) that stay on one XCD
-    if (kChunk > 0 && bid < (gridDim.x / (8u * kChunk)) * (8u * kChunk)) {
+    if (bid < (gridDim.x / (8u * run)) * (8u * run)) {
         const uint32_t local = bid >> 3;
-        bid = ((local / kChunk) * 8u + (bid & 7u)) * kChunk + local % kChunk;
+        bid = ((local / run) * 8u + (bid & 7u)) * run + local % run;
     }
     const uint32_t id = bid * kThreads + threadIdx.x;               // items < 2^31 (checked by the host)
     if (id >= items) return;
@@ -559,11 +562,13 @@ static int token_split_impl(const char *who, bool pair, const void *merged, cons
         COME_REQUIRE(items < (1ll << 31), COME_ERR_UNSUPPORTED, "%s: problem too large for one launch", who);
         const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
         const FastDiv by_out_chunks = make_fastdiv(out_chunks);
+        const int64_t run64 = static_cast<int64_t>(kSplitRunRows) * out_chunks / kThreads;
+        const uint32_t run = static_cast<uint32_t>(run64 < 1 ? 1 : (run64 > 4096 ? 4096 : run64));
         const uint4 *a4 = static_cast<const uint4 *>(merged), *b4 = static_cast<const uint4 *>(merged_b);
         uint4 *o4 = static_cast<uint4 *>(out);
 #define COME_SPLIT_CASE(IDX_, PAIR_, REV_)                                                                       \
     hipLaunchKernelGGL((split_vec_kernel<IDX_, PAIR_>), grid, block, 0, s, a4, b4, merged_rows, REV_, total,     \
-                       chunks, o4, items, by_out_chunks)
+                       chunks, o4, items, by_out_chunks, run)
         if (rev_i64 && pair) COME_SPLIT_CASE(int64_t, true, rev_i64);
         else if (rev_i64) COME_SPLIT_CASE(int64_t, false, rev_i64);
         else if (pair) COME_SPLIT_CASE(int32_t, true, rev_i32);
