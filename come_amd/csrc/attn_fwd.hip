@@ -704,12 +704,16 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
 }
 
 // Combines the key shares of the split query blocks: with m* the largest reference point of a row,
-// O = sum_i 2^(m_i - m*) O_i / sum_i 2^(m_i - m*) l_i.  One workgroup per split query block.
+// O = sum_i 2^(m_i - m*) O_i / sum_i 2^(m_i - m*) l_i.  One thread per (row, four output elements); a workgroup
+// covers 16 rows of a split query block, so the grid is (split query blocks) x block_m / 16 workgroups.
 template <int DT>
 __global__ __launch_bounds__(256) void attn_combine_kernel(const AttnArgs a, int block_m) {
     using E = Elem<DT>;
-    const int tail = blockIdx.x % a.nb_tail;
-    const int unit = blockIdx.x / a.nb_tail;
+    const int groups = block_m / 16;
+    const int group = blockIdx.x % groups;
+    const int block = blockIdx.x / groups;
+    const int tail = block % a.nb_tail;
+    const int unit = block / a.nb_tail;
     const int head = unit % a.n_heads;
     const int seq = unit / a.n_heads;
     int seq_start, L;
@@ -719,10 +723,11 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const AttnArgs a, int
     const int q0 = mblk * block_m;
     const int64_t piece_floats = static_cast<int64_t>(block_m) * (kHeadDim + kPieceExtra);
     const float *first = a.work + (static_cast<int64_t>(unit) * a.nb_tail + tail) * a.splits * piece_floats;
-    for (int idx = threadIdx.x; idx < block_m * (kHeadDim / 4); idx += blockDim.x) {
+    {
+        const int idx = group * 256 + threadIdx.x;
         const int local_row = idx / (kHeadDim / 4);
         const int c4 = idx % (kHeadDim / 4);
-        if (q0 + local_row >= L) continue;
+        if (q0 + local_row >= L) return;
         float m_star = -INFINITY;
         for (int i = 0; i < a.splits; ++i) {
             const float *pc = first + i * piece_floats;
@@ -885,7 +890,9 @@ extern "C" int come_attn_varlen_fwd_ws(const void *q, const void *k, const void 
     a.work = static_cast<float *>(work);
     a.n_full_wg = ceil_div(n_seq * n_heads, 8) * 8 * a.n_mblocks;
     const int64_t n_wg = a.n_full_wg + ceil_div(n_seq * n_heads, 8) * 8 * (plan.splits > 1 ? plan.nb_tail * plan.splits : 0);
-    COME_REQUIRE(n_wg < (1ll << 31), COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: grid too large");
+    const int64_t n_cwg = n_seq * n_heads * plan.nb_tail * (kBlockM / 16);       // combine kernel: 16 rows each
+    COME_REQUIRE(n_wg < (1ll << 31) && n_cwg < (1ll << 31), COME_ERR_UNSUPPORTED,
+                 "come_attn_varlen_fwd: grid too large");
     const dim3 grid(static_cast<unsigned>(n_wg)), block(wide ? 512 : 256);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (wide) {
@@ -897,7 +904,8 @@ extern "C" int come_attn_varlen_fwd_ws(const void *q, const void *k, const void 
     }
     COME_CHECK_LAUNCH("come_attn_varlen_fwd");
     if (plan.splits > 1) {
-        const dim3 cgrid(static_cast<unsigned>(n_seq * n_heads * plan.nb_tail));
+        static_assert(kHeadDim / 4 == 16, "a workgroup of the combine kernel covers 16 rows of 16 four-element chunks");
+        const dim3 cgrid(static_cast<unsigned>(n_cwg));
         if (dtype == COME_BF16) hipLaunchKernelGGL(attn_combine_kernel<COME_BF16>, cgrid, dim3(256), 0, s, a, kBlockM);
         else hipLaunchKernelGGL(attn_combine_kernel<COME_F16>, cgrid, dim3(256), 0, s, a, kBlockM);
         COME_CHECK_LAUNCH("come_attn_varlen_fwd (combine)");
