@@ -36,9 +36,9 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 # WRITE_SIZE passes (KiB per dispatch), FETCH_SIZE scaled by 2.000 and WRITE_SIZE by 1.000 -- the factors a 256 MiB
 # device copy (``--only copy``) gives for the same counters.  The summaries are in profiles/.
 TRAFFIC_BYTES = {
-    "attn": int((266761 * 2.000 + 97753) * 1024),
-    "merge": int((22066 * 2.000 + 25836) * 1024),
-    "unmerge": int((16126 * 2.000 + 44017) * 1024),
+    "attn": int((266700 * 2.000 + 97750) * 1024),
+    "merge": int((22070 * 2.000 + 25840) * 1024),
+    "unmerge": int((13570 * 2.000 + 43990) * 1024),
 }
 
 

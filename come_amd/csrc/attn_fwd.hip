@@ -127,25 +127,18 @@ __device__ inline void segment_of(const AttnArgs &a, int seq, int &seq_start, in
 // A split workgroup (behind the n_full_wg ordinary ones) gets the index of its query block among the unit's
 // tail blocks (tail >= 0) and its key share ks; the pieces of one query block are neighbours on one XCD.
 __device__ inline bool locate_block(const AttnArgs &a, int &mblk, int &head, int &seq, int &tail, int &ks) {
-    int unit;
-    if (static_cast<int64_t>(blockIdx.x) < a.n_full_wg) {
-        const int xcd = blockIdx.x & 7;
-        const int local = blockIdx.x >> 3;
-        unit = xcd + 8 * (local / a.n_mblocks);
-        mblk = local % a.n_mblocks;
-        tail = -1;
-        ks = 0;
-    } else {
-        const int e = static_cast<int>(blockIdx.x - a.n_full_wg);
-        const int xcd = e & 7;
-        const int local = e >> 3;
-        const int per_unit = a.nb_tail * a.splits;
-        unit = xcd + 8 * (local / per_unit);
-        const int within = local % per_unit;
-        tail = within / a.splits;
-        ks = within % a.splits;
-        mblk = 0;
-    }
+    // one straight-line computation for both kinds of workgroup (branches that assign different outputs made the
+    // compiler keep the outputs in scratch memory)
+    const bool split = static_cast<int64_t>(blockIdx.x) >= a.n_full_wg;
+    const int e = split ? static_cast<int>(blockIdx.x - a.n_full_wg) : static_cast<int>(blockIdx.x);
+    const int xcd = e & 7;
+    const int local = e >> 3;
+    const int per_unit = split ? a.nb_tail * a.splits : a.n_mblocks;
+    const int unit = xcd + 8 * (local / per_unit);
+    const int within = local % per_unit;
+    mblk = split ? 0 : within;
+    tail = split ? within / a.splits : -1;
+    ks = split ? within % a.splits : 0;
     head = unit % a.n_heads;
     seq = unit / a.n_heads;
     return unit < a.n_units;
