@@ -170,7 +170,8 @@ int64_t come_select_work_bytes(int64_t batch, int64_t frames, int64_t grid_h, in
  *   perkey_bias [total] of `dtype`, or NULL for plain attention
  *   max_seqlen  upper bound of the segment lengths (sizes the launch grid)
  *   out       [total, n_heads, head_dim] of `dtype`, strides in elements
- *   lse       [n_heads, total] float: logsumexp of the biased, scaled scores; may be NULL
+ *   lse       [n_heads, total] float: logsumexp of the biased, scaled scores (within 1e-2: the
+ *             scaled q is rounded to 16 bits); may be NULL
  * Only head_dim == 64 is implemented.  Probabilities are kept relative to a lazily moved reference point of
  * their row and stored in `dtype`: with COME_BF16 a key may exceed everything its row has seen so far by 2^87
  * within one 32-key step, with COME_F16 only by about 2^11 (7.6 nats) before the stored probability saturates at 65504 (the result

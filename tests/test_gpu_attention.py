@@ -280,3 +280,56 @@ def test_full_size_c3_rows_against_oracle_rows():
         diff = (out[row] - ref).abs()
         assert float(diff.max()) <= MAX_ABS and float(diff.mean()) <= MEAN_ABS
         torch.testing.assert_close(lse[:, row], torch.logsumexp(scores, -1), atol=2e-3, rtol=1e-3)
+
+
+BORDER_LENGTHS = [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 300, 511, 512, 513, 767, 769, 1023, 1025]
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_with_lengths_at_tile_borders(seed):
+    """Seeded sweep: segment lengths drawn from the borders of the 32 / 64-key tiles and the 256 / 512-query blocks,
+    1 to 6 segments (some empty), several head counts, both dtypes, bias kinds and scales; q, k, v either views
+    of one packed tensor or separate tensors with strides of their own; ``out_`` either fresh or supplied."""
+    g = torch.Generator().manual_seed(1000 + seed)
+    pick = lambda seq: seq[int(torch.randint(len(seq), (1,), generator=g))]
+    n_seq = pick([1, 2, 3, 4, 6])
+    lens = [pick(BORDER_LENGTHS + [0]) for _ in range(n_seq)]
+    if sum(lens) == 0:
+        lens[0] = 65
+    H = pick([1, 2, 3, 5, 16])
+    dtype = pick([torch.bfloat16, torch.bfloat16, torch.float16])
+    scale = pick([0.125, 0.1, 0.2])
+    P = sum(lens)
+    qkv = torch.randn(P, 3, H, 64, generator=g).to(dtype)
+    kind = pick(["counts", "weights", None])
+    if kind == "counts":
+        bias = torch.where(torch.rand(P, generator=g) < 0.3, math.log(9.0), 0.0).to(dtype)
+    elif kind == "weights":
+        bias = torch.rand(P, generator=g).clamp(min=1e-3).log().to(dtype)
+    else:
+        bias = None
+    cu = _cu(lens)
+    ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias, softmax_scale=scale)
+    max_len = max(lens)
+    if pick([True, False]):
+        q, k, v = qkv.to(DEV).unbind(1)                                            # views into the packed tensor
+    else:
+        pad = [torch.zeros(P, H, 64 + 8 * (i + 1), dtype=dtype, device=DEV) for i in range(3)]
+        for i in range(3):
+            pad[i][..., :64] = qkv[:, i].to(DEV)
+        q, k, v = (t[..., :64] for t in pad)                                         # three row / head strides
+    out_ = torch.full((P, H, 64), float("nan"), dtype=dtype, device=DEV) if pick([True, False]) else None
+    out, lse, _, _ = flash_attn_fwd_cuda.varlen_fwd_w_perkey_bias(
+        q, k, v, out_, cu.to(DEV), cu.to(DEV), None, None, None, None, None if bias is None else bias.to(DEV),
+        max_len, max_len, 0.0, scale, False, False, -1, -1, 0.0, False, None)
+    if out_ is not None:
+        assert out.data_ptr() == out_.data_ptr()
+    assert bool(torch.isfinite(out).all())
+    # short segments and sharp softmaxes (scale 0.2) give outputs of size 1 to 4, where rounding the result to 16
+    # bits alone costs up to 2^-9 of the value (2^-10 on average): the bounds are the reference's own
+    # (test_flex_attention_bias.py:20-21, atol = rtol = 1e-2) and the mean bound with that allowance
+    diff = (out.float().cpu() - ref).abs()
+    torch.testing.assert_close(out.float().cpu(), ref, atol=1e-2, rtol=1e-2)
+    assert float(diff.mean()) <= MEAN_ABS + 2.0 ** -9 * float(ref.abs().mean()), f"mean-abs {float(diff.mean())}"
+    # the kernel rounds the scaled Q to 16 bits: a logit, and with it lse, moves by up to 2^-9 of the logit's size
+    torch.testing.assert_close(lse.cpu(), ref_lse, atol=1e-2, rtol=1e-3)
