@@ -126,6 +126,17 @@ def co_me_token_split_pair_cuda(merged_a: torch.Tensor, merged_b: torch.Tensor, 
     return out
 
 
+def co_me_token_merge_cuda_legacy(*args, **kwargs):
+    """The reference still exports its first-generation pair (``co_me_cuext.pyi:22-46``) but calls it nowhere;
+    it is not provided here."""
+    raise RuntimeError("co_me_token_merge_cuda_legacy is not provided by the HIP build: use co_me_token_merge_cuda")
+
+
+def co_me_token_merge_scan_legacy(*args, **kwargs):
+    """See ``co_me_token_merge_cuda_legacy``."""
+    raise RuntimeError("co_me_token_merge_scan_legacy is not provided by the HIP build: use co_me_token_merge_cuda")
+
+
 def co_me_token_merge_2d_cuda(tokens: torch.Tensor, start_index: int, group_h: int, group_w: int, H: int, W: int,
                               merge_mask: torch.Tensor, index_dtype: torch.dtype = torch.int64,
                               count_dtype: torch.dtype = torch.float32):

@@ -43,3 +43,15 @@ def test_operators_refuse_cpu_tensors():
     cu = torch.tensor([0, 8], dtype=torch.int32)
     with pytest.raises(RuntimeError, match="CUDA"):
         flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, 8, perkey_bias=torch.zeros(8).bfloat16())
+
+
+def test_split_pair_and_legacy_entry_points_on_the_host():
+    from come_amd.cuda_extension import co_me_cuext
+    a = torch.randn(4, 8)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        co_me_cuext.co_me_token_split_pair_cuda(a, a, torch.zeros(3, dtype=torch.int64), 8)
+    # the reference exports a first-generation pair that nothing calls (co_me_cuext.pyi:22-46): refused by name
+    with pytest.raises(RuntimeError, match="not provided"):
+        co_me_cuext.co_me_token_merge_cuda_legacy(0, a, a, None)
+    with pytest.raises(RuntimeError, match="not provided"):
+        co_me_cuext.co_me_token_merge_scan_legacy(0, 2, a)
