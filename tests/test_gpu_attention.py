@@ -333,3 +333,31 @@ def test_random_shapes_with_lengths_at_tile_borders(seed):
     assert float(diff.mean()) <= MEAN_ABS + 2.0 ** -9 * float(ref.abs().mean()), f"mean-abs {float(diff.mean())}"
     # the kernel rounds the scaled Q to 16 bits: a logit, and with it lse, moves by up to 2^-9 of the logit's size
     torch.testing.assert_close(lse.cpu(), ref_lse, atol=1e-2, rtol=1e-3)
+
+
+def test_bias_of_minus_infinity_masks_keys():
+    """A caller may mask keys with a bias of -inf (the Co-Me path never does: log(count) >= 0).  Masked keys get
+    probability exactly 0, also when every one of the first keys of a segment - from which the kernel takes its
+    reference points - is masked."""
+    lens, H = [700, 90], 3
+    P = sum(lens)
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn(P, 3, H, 64, generator=g).bfloat16()
+    bias = torch.where(torch.rand(P, generator=g) < 0.3, -math.inf, 0.0)
+    bias[:40] = -math.inf                                              # the whole first 32-key step of segment 0
+    bias[40] = 0.0
+    bias[700:730] = -math.inf                                          # most of the first step of segment 1
+    bias = bias.bfloat16()
+    cu = _cu(lens)
+    ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias)
+    assert bool(torch.isfinite(ref).all())
+    out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), 700, perkey_bias=bias.to(DEV),
+                                                                 return_attn_probs=True)
+    assert bool(torch.isfinite(out).all())
+    _compare(out, ref)
+    torch.testing.assert_close(lse.cpu(), ref_lse, atol=1e-2, rtol=1e-3)
+    # a masked key cannot reach the output: changing its value row changes nothing, bit for bit
+    qkv2 = qkv.clone()
+    qkv2[:40, 2] = 1000.0
+    out2 = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv2.to(DEV), cu.to(DEV), 700, perkey_bias=bias.to(DEV))
+    assert torch.equal(out2, out)
