@@ -164,10 +164,13 @@ def jittered_frame_masks(conf, ratio, jitter, seed):
     return rank < k[:, None]
 
 
-def merge_workload(device, ratio=0.5, sets=8, frames=16, H=37, W=37, jitter=None, dtype=None, C=1024):
-    """Merge microbenchmark: 16 frames, 37x37 patches + 5 specials, C = 1024, bf16.  ``sets`` rotating
-    input / output buffer sets keep the working set (> 500 MB) out of the 256 MB Infinity Cache.  With ``jitter``
-    the mask comes from ``jittered_frame_masks`` instead of the joint quantile selection."""
+def merge_workload(device, ratio=0.5, sets=None, frames=16, H=37, W=37, jitter=None, dtype=None, C=1024):
+    """Merge microbenchmark: 16 frames, 37x37 patches + 5 specials, C = 1024, bf16, over rotating input / output
+    buffer sets.  Every stream has to come from HBM, not from the 256 MB Infinity Cache, so the sets of each tensor a
+    kernel reads must exceed the cache on their own: ``sets=None`` takes as many as bring the packed rows (the
+    smallest stream, read by the unmerge) to 320 MB, at least 8.  (With 8 sets = 209 MB of packed rows at ratio 0.5
+    the unmerge read them from the cache and measured 6.2 instead of 4.7 TB/s.)  With ``jitter`` the mask comes from
+    ``jittered_frame_masks`` instead of the joint quantile selection."""
     import torch
     from come_amd import _lib
 
@@ -177,8 +180,6 @@ def merge_workload(device, ratio=0.5, sets=8, frames=16, H=37, W=37, jitter=None
     code, esize = _lib.dtype_code(dtype), torch.empty(0, dtype=dtype).element_size()
     lib = _lib.load()
     conf = smooth_confidence(frames, H, W, seed=0).to(device)
-    torch.manual_seed(0)
-    tokens = [torch.randn(frames, N, C, device=device).to(dtype) for _ in range(sets)]
     M = (H // 3) * (W // 3)
     tail = H * W - M * 9
     mask = torch.empty(frames, M, dtype=torch.uint8, device=device)
@@ -199,6 +200,11 @@ def merge_workload(device, ratio=0.5, sets=8, frames=16, H=37, W=37, jitter=None
 
     select_and_plan()
     P = int(offsets[-1].item())
+    if sets is None:
+        packed_bytes = P * C * esize
+        sets = 2 if packed_bytes < (1 << 20) else max(8, -(-320_000_000 // packed_bytes))
+    torch.manual_seed(0)
+    tokens = [torch.randn(frames, N, C, device=device).to(dtype) for _ in range(sets)]
     outs = [torch.empty(P, C, dtype=dtype, device=device) for _ in range(sets)]
     index_map = torch.empty(frames * N, dtype=torch.int32, device=device)
     counts = torch.empty(P, dtype=torch.int32, device=device)
@@ -231,7 +237,7 @@ def merge_workload(device, ratio=0.5, sets=8, frames=16, H=37, W=37, jitter=None
 
 def bench_merge_unmerge(device, iters=200, warmup=20):
     w = merge_workload(device)
-    for _ in range(8):
+    for _ in range(len(w["outs"])):
         w["merge_only"]()                                       # fill every output set before unmerge reads it
     _, merge_ms = time_loop(w["merge_only"], iters, warmup)
     _, pipe_ms = time_loop(w["pipeline"], iters, warmup)
@@ -241,13 +247,13 @@ def bench_merge_unmerge(device, iters=200, warmup=20):
     return w, {
         "merge": {"workload": "C2 merge: 16 frames 37x37+5, C=1024 bf16, 3x3, ratio 0.5, P=%d" % w["P"],
                   "value": round(merge_gbs, 1), "unit": "GB/s", "us_per_call": round(merge_ms / iters * 1e3, 2),
-                  "algorithmic_bytes": w["merge_bytes"], "iters": iters, "rotating_buffer_sets": 8,
+                  "algorithmic_bytes": w["merge_bytes"], "iters": iters, "rotating_buffer_sets": len(w["outs"]),
                   "roofline": {"bound": "hbm", "achieved": round(merge_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                "frac": round(merge_gbs / PEAK_HBM_GBS, 4), "traffic": TRAFFIC_BYTES["merge"]},
                   "select_plan_merge_us": round(pipe_ms / iters * 1e3, 2)},
         "unmerge": {"workload": "C2 unmerge: P=%d -> %d rows, C=1024 bf16" % (w["P"], w["frames"] * w["N"]),
                     "value": round(split_gbs, 1), "unit": "GB/s", "us_per_call": round(split_ms / iters * 1e3, 2),
-                    "algorithmic_bytes": w["split_bytes"], "iters": iters, "rotating_buffer_sets": 8,
+                    "algorithmic_bytes": w["split_bytes"], "iters": iters, "rotating_buffer_sets": len(w["outs"]),
                     "roofline": {"bound": "hbm", "achieved": round(split_gbs, 1), "peak": PEAK_HBM_GBS,
                                  "unit": "GB/s", "frac": round(split_gbs / PEAK_HBM_GBS, 4),
                                  "traffic": TRAFFIC_BYTES["unmerge"]}},
@@ -261,10 +267,8 @@ def bench_merge_caller_dtypes(device, iters=200, warmup=20):
 
     out = {}
     for name, dtype, C in (("fp32_c1024", torch.float32, 1024), ("bf16_c2", torch.bfloat16, 2)):
-        # 4 rotating sets of the fp32 tensors have the footprint (570 MB) of the 8 bf16 sets of the headline
-        # microbenchmark; the unmerge rate falls off beyond about 1 GB of rotating buffers (8 fp32 sets: 5.4 TB/s)
-        w = merge_workload(device, dtype=dtype, C=C, sets=4 if C > 2 else 2)
-        for _ in range(4):
+        w = merge_workload(device, dtype=dtype, C=C)
+        for _ in range(len(w["outs"])):
             w["merge_only"]()
         _, m_ms = time_loop(w["merge_only"], iters, warmup)
         _, s_ms = time_loop(w["split_only"], iters, warmup)
@@ -319,7 +323,7 @@ def bench_merge_ratios(device, iters=200, warmup=20):
     out = {}
     for ratio in (0.25, 0.75):
         w = merge_workload(device, ratio=ratio)
-        for _ in range(8):
+        for _ in range(len(w["outs"])):
             w["merge_only"]()
         _, m_ms = time_loop(w["merge_only"], iters, warmup)
         _, s_ms = time_loop(w["split_only"], iters, warmup)
@@ -375,10 +379,8 @@ def bench_stress(device):
     tokens), 3x3 merge at ratio 0.75 with per-frame jitter +-0.1."""
     import torch
 
-    # two rotating sets of 376 MB each: every launch moves more than the 256 MB Infinity Cache holds; with three sets
-    # (1.1 GB of rotating buffers) the unmerge rate drops from 7.0 to 4.9 TB/s, the merge rate stays
-    w = merge_workload(device, ratio=0.75, sets=2, frames=128, H=37, W=28, jitter=0.1)
-    for _ in range(2):
+    w = merge_workload(device, ratio=0.75, sets=4, frames=128, H=37, W=28, jitter=0.1)   # 4 x 102 MB of packed rows
+    for _ in range(4):
         w["merge_only"]()
     _, m_ms = time_loop(w["merge_only"], 50, 10)
     _, s_ms = time_loop(w["split_only"], 50, 10)
@@ -390,7 +392,7 @@ def bench_stress(device):
            "merge_us": round(m_ms / 50 * 1e3, 1), "merge_bytes": w["merge_bytes"],
            "merge_GBs": round(w["merge_bytes"] / (m_ms / 50 * 1e-3) / 1e9, 1),
            "unmerge_us": round(s_ms / 50 * 1e3, 1), "unmerge_bytes": w["split_bytes"],
-           "unmerge_GBs": round(w["split_bytes"] / (s_ms / 50 * 1e-3) / 1e9, 1), "rotating_buffer_sets": 2}
+           "unmerge_GBs": round(w["split_bytes"] / (s_ms / 50 * 1e-3) / 1e9, 1), "rotating_buffer_sets": 4}
     P = w["P"]
     del w
     torch.cuda.empty_cache()
@@ -564,12 +566,12 @@ def main():
             print(json.dumps({"only": "dtypes", **bench_merge_caller_dtypes(device, args.steps, args.warmup)}))
         elif args.only == "pair":
             mw = merge_workload(device)
-            for _ in range(8):
+            for _ in range(len(mw["outs"])):
                 mw["merge_only"]()
             print(json.dumps({"only": "pair", **bench_unmerge_pair(device, mw, args.steps, args.warmup)}))
         else:
             mw = merge_workload(device)
-            for _ in range(8):
+            for _ in range(len(mw["outs"])):
                 mw["merge_only"]()
             fn = mw["merge_only"] if args.only == "merge" else mw["split_only"]
             _, ms = time_loop(fn, args.steps, args.warmup)

@@ -13,6 +13,12 @@ namespace come {
 namespace {
 
 constexpr int kThreads = 256;
+#ifndef COME_MERGE_THREADS
+#define COME_MERGE_THREADS 64
+#endif
+// the 16-byte merge kernel runs one wavefront per workgroup (measured at 64 / 128 / 256 / 512 / 1024 threads on the
+// 16-frame microbenchmark: 14.2 / 14.6 / 14.8 / 16.0 / 18.1 us)
+constexpr int kMergeThreads = COME_MERGE_THREADS;
 
 // 16-byte global accesses; the streamed variants carry the non-temporal hint (data used once)
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -150,7 +156,7 @@ __global__ __launch_bounds__(1024) void merge_plan_kernel(const uint8_t *__restr
 // merge, 16-byte path.  GH x GW fixed at compile time (0 x 0 = run-time window shape).
 // ---------------------------------------------------------------------------------
 template <int DT, int GH, int GW>
-__global__ __launch_bounds__(kThreads) void merge_vec_kernel(const MergeArgs a) {
+__global__ __launch_bounds__(kMergeThreads) void merge_vec_kernel(const MergeArgs a) {
     using V = Vec16<DT>;
     const MergeGeom &g = a.g;
     const uint4 *__restrict__ src = static_cast<const uint4 *>(a.tokens);
@@ -158,7 +164,7 @@ __global__ __launch_bounds__(kThreads) void merge_vec_kernel(const MergeArgs a) 
     const int chunks = a.chunks;
 
     if (static_cast<int64_t>(blockIdx.x) < a.group_blocks) {
-        const uint32_t id = blockIdx.x * kThreads + threadIdx.x;     // item counts stay below 2^31 (checked by the host)
+        const uint32_t id = blockIdx.x * kMergeThreads + threadIdx.x;     // item counts stay below 2^31 (checked by the host)
         if (id >= a.group_items) return;
         const uint32_t gm = fast_div(id, a.by_chunks);      // flat (row, window)
         const int chunk = static_cast<int>(id - gm * chunks);
@@ -238,7 +244,7 @@ __global__ __launch_bounds__(kThreads) void merge_vec_kernel(const MergeArgs a) 
     }
 
     // copied tokens: specials in front, leftover grid positions behind the windows
-    const uint32_t id = (blockIdx.x - static_cast<uint32_t>(a.group_blocks)) * kThreads + threadIdx.x;
+    const uint32_t id = (blockIdx.x - static_cast<uint32_t>(a.group_blocks)) * kMergeThreads + threadIdx.x;
     if (id >= a.single_items) return;
     const int per_row = g.start + g.tail;
     const uint32_t t = fast_div(id, a.by_chunks);
@@ -337,7 +343,10 @@ __global__ __launch_bounds__(kThreads) void merge_elem_kernel(const MergeArgs a)
 // ---------------------------------------------------------------------------------
 // unmerge: out[i, :] = merged[rev[i], :]
 // ---------------------------------------------------------------------------------
-constexpr int kSplitRows = 1;      // output rows per thread (measured best of 1, 2, 3, 4, 8)
+#ifndef COME_SPLIT_ROWS
+#define COME_SPLIT_ROWS 1
+#endif
+constexpr int kSplitRows = COME_SPLIT_ROWS;      // output rows per thread (measured best of 1, 2, 3, 4, 8)
 #ifndef COME_SPLIT_RUN_ROWS
 #define COME_SPLIT_RUN_ROWS 256
 #endif
@@ -373,12 +382,20 @@ __global__ __launch_bounds__(kThreads) void split_vec_kernel(const uint4 *__rest
         v[r] = make_uint4(0, 0, 0, 0);
         if (i0 + r < total) {
             const int64_t s = static_cast<int64_t>(rev[i0 + r]);
+#if COME_SPLIT_LOAD_NT
+            if (s >= 0 && s < merged_rows) v[r] = ld16_stream(src + s * chunks + chunk);
+#else
             if (s >= 0 && s < merged_rows) v[r] = src[s * chunks + chunk];
+#endif
         }
     }
 #pragma unroll
     for (int r = 0; r < kSplitRows; ++r)
+#if COME_SPLIT_STORE_PLAIN
+        if (i0 + r < total) out[(i0 + r) * out_chunks + out_chunk] = v[r];
+#else
         if (i0 + r < total) st16_stream(out + (i0 + r) * out_chunks + out_chunk, v[r]);
+#endif
 }
 
 // element-wise fallback; `pair`: output rows are [row of merged | row of merged_b]
@@ -410,7 +427,7 @@ __global__ __launch_bounds__(kThreads) void split_elem_kernel(const uint8_t *__r
 template <int DT>
 void launch_merge_vec(const MergeArgs &a, int64_t blocks, hipStream_t stream) {
     const MergeGeom &g = a.g;
-    const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+    const dim3 grid(static_cast<unsigned>(blocks)), block(kMergeThreads);
 #define COME_MERGE_CASE(GH_, GW_)                                                              \
     if (g.gh == GH_ && g.gw == GW_) {                                                          \
         hipLaunchKernelGGL((merge_vec_kernel<DT, GH_, GW_>), grid, block, 0, stream, a);       \
@@ -512,7 +529,8 @@ extern "C" int come_token_merge(const void *tokens, int dtype, int64_t rows, int
     const bool vec = (row_bytes % 16 == 0) && aligned16(tokens) && aligned16(out);
     a.chunks = static_cast<int>(vec ? row_bytes / 16 : chans);
     a.group_items = rows * g.groups * a.chunks;
-    a.group_blocks = ceil_div(a.group_items, kThreads);
+    const int threads = vec ? kMergeThreads : kThreads;
+    a.group_blocks = ceil_div(a.group_items, threads);
     a.single_items = rows * (g.start + g.tail) * a.chunks;
     COME_REQUIRE(!vec || (a.group_items < (1ll << 31) && a.single_items < (1ll << 31)), COME_ERR_UNSUPPORTED,
                  "come_token_merge: more than 2^31 16-byte items in one launch");
@@ -521,7 +539,7 @@ extern "C" int come_token_merge(const void *tokens, int dtype, int64_t rows, int
     a.by_mw = make_fastdiv(g.mw > 0 ? g.mw : 1);
     a.by_per_row = make_fastdiv(g.start + g.tail > 0 ? g.start + g.tail : 1);
     a.by_side = make_fastdiv(g.W - g.cov_w > 0 ? g.W - g.cov_w : 1);
-    const int64_t blocks = a.group_blocks + ceil_div(a.single_items, kThreads);
+    const int64_t blocks = a.group_blocks + ceil_div(a.single_items, threads);
     COME_REQUIRE(blocks < (1ll << 31), COME_ERR_UNSUPPORTED, "come_token_merge: problem too large for one launch");
     if (blocks == 0) return COME_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
