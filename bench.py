@@ -37,8 +37,8 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 # device copy (``--only copy``) gives for the same counters.  The summaries are in profiles/.
 TRAFFIC_BYTES = {
     "attn": int((266700 * 2.000 + 97750) * 1024),
-    "merge": int((22070 * 2.000 + 25840) * 1024),
-    "unmerge": int((13570 * 2.000 + 43990) * 1024),
+    "merge": int((22070 * 2.000 + 25940) * 1024),
+    "unmerge": int((13570 * 2.000 + 43970) * 1024),
 }
 
 
