@@ -13,12 +13,9 @@ namespace come {
 namespace {
 
 constexpr int kThreads = 256;
-#ifndef COME_MERGE_THREADS
-#define COME_MERGE_THREADS 64
-#endif
 // the 16-byte merge kernel runs one wavefront per workgroup (measured at 64 / 128 / 256 / 512 / 1024 threads on the
 // 16-frame microbenchmark: 14.2 / 14.6 / 14.8 / 16.0 / 18.1 us)
-constexpr int kMergeThreads = COME_MERGE_THREADS;
+constexpr int kMergeThreads = 64;
 
 // 16-byte global accesses; the streamed variants carry the non-temporal hint (data used once)
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -343,14 +340,8 @@ __global__ __launch_bounds__(kThreads) void merge_elem_kernel(const MergeArgs a)
 // ---------------------------------------------------------------------------------
 // unmerge: out[i, :] = merged[rev[i], :]
 // ---------------------------------------------------------------------------------
-#ifndef COME_SPLIT_ROWS
-#define COME_SPLIT_ROWS 1
-#endif
-constexpr int kSplitRows = COME_SPLIT_ROWS;      // output rows per thread (measured best of 1, 2, 3, 4, 8)
-#ifndef COME_SPLIT_RUN_ROWS
-#define COME_SPLIT_RUN_ROWS 256
-#endif
-constexpr int kSplitRunRows = COME_SPLIT_RUN_ROWS;   // output rows that stay on one XCD
+constexpr int kSplitRows = 1;         // output rows per thread (measured best of 1, 2, 3, 4, 8)
+constexpr int kSplitRunRows = 256;    // output rows that stay on one XCD (64 - 1024 measured: no difference)
 
 // PAIR: two packed sources with one index map; an output row holds the row of `merged` followed by the row of
 // `merged_b` (`chunks` is the width of one source row, an output row has 2 * chunks chunks).
@@ -382,20 +373,12 @@ __global__ __launch_bounds__(kThreads) void split_vec_kernel(const uint4 *__rest
         v[r] = make_uint4(0, 0, 0, 0);
         if (i0 + r < total) {
             const int64_t s = static_cast<int64_t>(rev[i0 + r]);
-#if COME_SPLIT_LOAD_NT
-            if (s >= 0 && s < merged_rows) v[r] = ld16_stream(src + s * chunks + chunk);
-#else
             if (s >= 0 && s < merged_rows) v[r] = src[s * chunks + chunk];
-#endif
         }
     }
 #pragma unroll
     for (int r = 0; r < kSplitRows; ++r)
-#if COME_SPLIT_STORE_PLAIN
-        if (i0 + r < total) out[(i0 + r) * out_chunks + out_chunk] = v[r];
-#else
         if (i0 + r < total) st16_stream(out + (i0 + r) * out_chunks + out_chunk, v[r]);
-#endif
 }
 
 // element-wise fallback; `pair`: output rows are [row of merged | row of merged_b]
