@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "copy", "e2e", "stress", "stress_e2e", "frame"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "copy", "e2e", "stress", "stress_e2e", "frame"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -359,6 +359,32 @@ def attention_case(device, lens, counts, steps, warmup, H=16, D=64):
     return ms / steps, flops / (ms / steps * 1e-3) / 1e12, flops
 
 
+def bench_bias_overhead(device):
+    """What the reference's own microbenchmark checks (test/benchmark/bench_flash_attn_w_bias.py: the per-key bias
+    must cost next to nothing over the plain kernel): its head_dim 64, non-causal shapes and the headline shape,
+    with and without bias."""
+    import torch
+    from come_amd.cuda_extension import (flash_attn_varlen_qkvpacked_func,
+                                         flash_attn_varlen_qkvpacked_func_w_perkey_bias)
+
+    out = {}
+    shapes = (("tiny b=4 s=128 h=8 fp16", [128] * 4, 8, torch.float16), ("small b=8 s=256 h=16 fp16", [256] * 8, 16, torch.float16),
+              ("small b=8 s=256 h=16 bf16", [256] * 8, 16, torch.bfloat16), ("headline L={25536,21848} h=16 bf16", [25536, 21848], 16, torch.bfloat16))
+    for name, lens, H, dtype in shapes:
+        P = sum(lens)
+        torch.manual_seed(2)
+        qkv = torch.randn(P, 3, H, 64, device=device).to(dtype)
+        bias = (torch.randn(P, device=device) * 0.1).to(dtype)
+        cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=device)
+        steps = 200 if P < 10000 else 10
+        _, plain_ms = time_loop(lambda: flash_attn_varlen_qkvpacked_func(qkv, cu, max(lens)), steps, 5)
+        _, bias_ms = time_loop(lambda: flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, max(lens), perkey_bias=bias),
+                               steps, 5)
+        out[name] = {"plain_us": round(plain_ms / steps * 1e3, 2), "with_bias_us": round(bias_ms / steps * 1e3, 2),
+                     "ratio": round(plain_ms / bias_ms, 4)}
+    return out
+
+
 def bench_frame_attention(device, w):
     """Frame-mode attention of the headline workload's first sequence: 32 segments of about 798 tokens."""
     import torch
@@ -562,6 +588,8 @@ def main():
             w, wall, ev_ms = bench_attention(args.steps, args.warmup, device)
             print(json.dumps({"only": "attn", "ms_per_call": ev_ms / args.steps,
                               "tflops": w["flops"] / (ev_ms / args.steps * 1e-3) / 1e12}))
+        elif args.only == "bias":
+            print(json.dumps({"only": "bias", **bench_bias_overhead(device)}))
         elif args.only == "dtypes":
             print(json.dumps({"only": "dtypes", **bench_merge_caller_dtypes(device, args.steps, args.warmup)}))
         elif args.only == "pair":
@@ -615,6 +643,7 @@ def main():
         other["merge_other_ratios"] = bench_merge_ratios(device)
         other["merge_caller_dtypes"] = bench_merge_caller_dtypes(device)
         other["frame_attention"] = bench_frame_attention(device, w)
+        other["bias_overhead"] = bench_bias_overhead(device)
         other["stress"] = bench_stress(device)
     if not args.no_e2e:
         result.setdefault("other", {})["e2e"] = bench_e2e(device)

@@ -31,29 +31,40 @@ def _pad_head(t: torch.Tensor, head_size: int) -> torch.Tensor:
     return t
 
 
-class _VarlenQKVPacked(torch.autograd.Function):
+def _forward(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale, causal, window_size, softcap,
+             alibi_slopes, return_softmax):
     """Shared forward of the plain and the biased operator (``perkey_bias`` may be None)."""
+    if softmax_scale is None:
+        softmax_scale = qkv.shape[-1] ** (-0.5)
+    if len(window_size) != 2:
+        raise ValueError(f"window_size must contain 2 values, got {window_size}")
+    q, k, v = qkv[:, 0].detach(), qkv[:, 1].detach(), qkv[:, 2].detach()
+    head_size_og = q.size(2)
+    if head_size_og % 8 != 0:
+        q, k, v = (_pad_head(t, head_size_og) for t in (q, k, v))
+    args = (q, k, v, None, cu_seqlens, cu_seqlens, None, None, None, alibi_slopes)
+    tail = (max_seqlen, max_seqlen, dropout_p, softmax_scale, False, causal, int(window_size[0]),
+            int(window_size[1]), softcap, return_softmax and dropout_p > 0, None)
+    if perkey_bias is None:
+        out_padded, softmax_lse, s_dmask, rng_state = _C.varlen_fwd(*args, *tail)
+    else:
+        out_padded, softmax_lse, s_dmask, rng_state = _C.varlen_fwd_w_perkey_bias(*args, perkey_bias, *tail)
+    out = out_padded if out_padded.shape[-1] == head_size_og else out_padded[..., :head_size_og]
+    return out, softmax_lse, s_dmask, rng_state
+
+
+class _VarlenQKVPacked(torch.autograd.Function):
+    """Records the operator in the autograd graph so that a backward pass raises, as in the reference
+    (``flash_attn/__init__.py:194-200, 398-403``).  Only used when an input requires a gradient."""
 
     @staticmethod
     def forward(ctx, qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale, causal, window_size,
                 softcap, alibi_slopes, deterministic, return_softmax, is_grad_enabled, op_name):
         ctx.op_name = op_name
-        if softmax_scale is None:
-            softmax_scale = qkv.shape[-1] ** (-0.5)
-        if len(window_size) != 2:
-            raise ValueError(f"window_size must contain 2 values, got {window_size}")
-        q, k, v = qkv[:, 0].detach(), qkv[:, 1].detach(), qkv[:, 2].detach()
-        head_size_og = q.size(2)
-        q, k, v = (_pad_head(t, head_size_og) for t in (q, k, v))
-        args = (q, k, v, None, cu_seqlens, cu_seqlens, None, None, None, alibi_slopes)
-        tail = (max_seqlen, max_seqlen, dropout_p, softmax_scale, False, causal, int(window_size[0]),
-                int(window_size[1]), softcap, return_softmax and dropout_p > 0, None)
-        if perkey_bias is None:
-            out_padded, softmax_lse, s_dmask, rng_state = _C.varlen_fwd(*args, *tail)
-        else:
-            out_padded, softmax_lse, s_dmask, rng_state = _C.varlen_fwd_w_perkey_bias(*args, perkey_bias, *tail)
+        out, softmax_lse, s_dmask, rng_state = _forward(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p,
+                                                        softmax_scale, causal, window_size, softcap, alibi_slopes,
+                                                        return_softmax)
         ctx.mark_non_differentiable(softmax_lse, s_dmask, rng_state)
-        out = out_padded[..., :head_size_og]
         return out if not return_softmax else (out, softmax_lse, s_dmask)
 
     @staticmethod
@@ -61,14 +72,27 @@ class _VarlenQKVPacked(torch.autograd.Function):
         raise RuntimeError(f"{ctx.op_name} backward is not supported in this forward-only build.")
 
 
+def _call(op_name, qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale, causal, window_size, softcap,
+          alibi_slopes, deterministic, return_attn_probs):
+    needs_graph = torch.is_grad_enabled() and (qkv.requires_grad
+                                               or (perkey_bias is not None and perkey_bias.requires_grad))
+    if needs_graph:
+        return _VarlenQKVPacked.apply(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale, causal,
+                                      window_size, softcap, alibi_slopes, deterministic, return_attn_probs, True,
+                                      op_name)
+    # inference: nothing to record, skip the autograd.Function machinery (about 10 us of host time per call)
+    out, softmax_lse, s_dmask, _ = _forward(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale,
+                                            causal, window_size, softcap, alibi_slopes, return_attn_probs)
+    return out if not return_attn_probs else (out, softmax_lse, s_dmask)
+
+
 def flash_attn_varlen_qkvpacked_func(qkv, cu_seqlens, max_seqlen, dropout_p=0.0, softmax_scale=None, causal=False,
                                      window_size=(-1, -1), softcap=0.0, alibi_slopes=None, deterministic=False,
                                      return_attn_probs=False):
     """``qkv [total, 3, nheads, headdim]``, ``cu_seqlens [batch + 1] int32`` -> ``out [total, nheads, headdim]``
     (plus ``softmax_lse [nheads, total]`` and an empty tensor when ``return_attn_probs``)."""
-    return _VarlenQKVPacked.apply(qkv, cu_seqlens, max_seqlen, None, dropout_p, softmax_scale, causal, window_size,
-                                  softcap, alibi_slopes, deterministic, return_attn_probs, torch.is_grad_enabled(),
-                                  "flash_attn_varlen_qkvpacked_func")
+    return _call("flash_attn_varlen_qkvpacked_func", qkv, cu_seqlens, max_seqlen, None, dropout_p, softmax_scale,
+                 causal, window_size, softcap, alibi_slopes, deterministic, return_attn_probs)
 
 
 def flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p=0.0,
@@ -77,6 +101,5 @@ def flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu_seqlens, max_seqlen, 
                                                    return_attn_probs=False):
     """Same as :func:`flash_attn_varlen_qkvpacked_func` with ``softmax(Q K^T * scale + perkey_bias[key]) V``;
     ``perkey_bias [total]`` has the dtype of ``qkv`` and is indexed like the packed keys."""
-    return _VarlenQKVPacked.apply(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale, causal,
-                                  window_size, softcap, alibi_slopes, deterministic, return_attn_probs,
-                                  torch.is_grad_enabled(), "flash_attn_varlen_qkvpacked_func_w_perkey_bias")
+    return _call("flash_attn_varlen_qkvpacked_func_w_perkey_bias", qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p,
+                 softmax_scale, causal, window_size, softcap, alibi_slopes, deterministic, return_attn_probs)

@@ -28,6 +28,35 @@ def _unsupported(cond: bool, what: str) -> None:
         raise RuntimeError(f"come_amd flash-attention: {what} is not supported by this forward-only HIP build")
 
 
+class _on_device:
+    """``torch.cuda.device(dev)`` that costs nothing when ``dev`` already is the current device."""
+
+    def __init__(self, dev: torch.device):
+        self.guard = None if dev.index is None or dev.index == torch.cuda.current_device() else torch.cuda.device(dev)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            return self.guard.__exit__(*exc)
+        return False
+
+
+_PLACEHOLDERS: dict = {}
+
+
+def _placeholders(dev: torch.device, dtype: torch.dtype):
+    """The two results the forward never fills (attention probabilities, dropout RNG state): one empty tensor
+    and one two-element int64 tensor per device and dtype, never written by anything in this package."""
+    key = (dev, dtype)
+    if key not in _PLACEHOLDERS:
+        _PLACEHOLDERS[key] = (torch.empty((0,), dtype=dtype, device=dev),
+                              torch.zeros((2,), dtype=torch.int64, device=dev))
+    return _PLACEHOLDERS[key]
+
+
 def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
                      perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal,
                      window_size_left, window_size_right, softcap, return_softmax, gen):
@@ -37,7 +66,8 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
     _check(cu_seqlens_q.dtype == torch.int32, "cu_seqlens_q must have dtype int32")
     _check(cu_seqlens_k.dtype == torch.int32, "cu_seqlens_k must have dtype int32")
     for name, t in (("q", q), ("k", k), ("v", v), ("cu_seqlens_q", cu_seqlens_q), ("cu_seqlens_k", cu_seqlens_k)):
-        _check(t.is_cuda, f"{name} must be on CUDA")
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} must be on CUDA")
     _check(q.stride(-1) == 1 and k.stride(-1) == 1 and v.stride(-1) == 1,
            "Input tensor must have contiguous last dimension")
     _check(cu_seqlens_q.is_contiguous() and cu_seqlens_k.is_contiguous(), "cu_seqlens must be contiguous")
@@ -71,25 +101,26 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
     _check(tuple(v.shape) == (total_k, num_heads_k, head_size), "v must have shape (total_k, num_heads_k, head_size)")
     _check(tuple(cu_seqlens_k.shape) == (batch_size + 1,), "cu_seqlens_k must have shape (batch_size + 1)")
     _unsupported(num_heads != num_heads_k, "grouped-query attention (num_heads != num_heads_k)")
-    _unsupported(head_size != 64, f"head_dim {head_size} (only 64 is implemented)")
+    if head_size != 64:
+        _unsupported(True, f"head_dim {head_size} (only 64 is implemented)")
     _unsupported(total_q != total_k or max_seqlen_q != max_seqlen_k
                  or (cu_seqlens_q.data_ptr() != cu_seqlens_k.data_ptr() and not torch.equal(cu_seqlens_q, cu_seqlens_k)),
                  "cross attention (different query and key packing)")
 
     dev = q.device
     if perkey_bias is not None:
-        _check(perkey_bias.dtype == q.dtype,
-               f"perkey_bias dtype must match QKV dtype ({q.dtype}), got {perkey_bias.dtype}")
+        if perkey_bias.dtype != q.dtype:
+            raise RuntimeError(f"perkey_bias dtype must match QKV dtype ({q.dtype}), got {perkey_bias.dtype}")
         _check(perkey_bias.is_cuda, "perkey_bias must be on CUDA")
         _check(perkey_bias.is_contiguous(), "perkey_bias must be contiguous")
-        _check(tuple(perkey_bias.shape) == (total_k,),
-               f"perkey_bias must have shape (total_k,), got {tuple(perkey_bias.shape)}")
+        if perkey_bias.dim() != 1 or perkey_bias.shape[0] != total_k:
+            raise RuntimeError(f"perkey_bias must have shape (total_k,), got {tuple(perkey_bias.shape)}")
 
     def _aligned(t):          # the kernel issues 16-byte loads
         return t.data_ptr() % 16 == 0 and t.stride(0) % 8 == 0 and t.stride(1) % 8 == 0
     q, k, v = (t if _aligned(t) else t.contiguous() for t in (q, k, v))
 
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         if out_ is not None:
             out = out_
             _check(out.dtype == q.dtype, "Output must have the same dtype as inputs")
@@ -99,8 +130,7 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
         else:
             out = torch.empty((total_q, num_heads, head_size), dtype=q.dtype, device=dev)
         softmax_lse = torch.empty((num_heads, total_q), dtype=torch.float32, device=dev)
-        p = torch.empty((0,), dtype=q.dtype, device=dev)
-        rng_state = torch.empty((2,), dtype=torch.int64, device=dev)
+        p, rng_state = _placeholders(dev, q.dtype)
         if zero_tensors:
             out.zero_()
             softmax_lse.fill_(-math.inf)

@@ -224,3 +224,38 @@ def test_split_pair_full_size_through_the_merger():
     assert both.shape == (B, S + H * W, 2 * C)
     assert torch.equal(both[..., :C], func_token_split(jag, rev, shape))
     assert torch.equal(both[..., C:], func_token_split(other, rev, shape))
+
+
+def test_operators_run_on_the_current_stream():
+    """The reference launches merge / split on the default stream whatever the caller's stream is
+    (kernel_token_merge.cu:275); here every operator is enqueued on torch's current stream.  The inputs are
+    produced on a side stream behind a few milliseconds of matrix products, so an operator that ran on another
+    stream would read them before they exist."""
+    from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
+    B, H, W, S, C = 4, 36, 36, 5, 256
+    g = torch.Generator().manual_seed(3)
+    tokens_cpu = torch.randn(B, S + H * W, C, generator=g).bfloat16()
+    mask_cpu = torch.rand(B, 144, generator=g) < 0.5
+    ref, ref_rev = oracle.token_merge_2d(tokens_cpu, S, 3, 3, H, W, mask_cpu)
+    src, mask = tokens_cpu.to(DEV), mask_cpu.to(DEV)
+    big = torch.randn(4096, 4096, device=DEV)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        acc = big
+        for _ in range(20):
+            acc = (acc @ big) * 1e-2                                    # a few milliseconds of work on the side stream
+        tokens = torch.zeros_like(src)
+        tokens += src + (acc[0, 0] * 0).to(src.dtype)                    # written behind the products, on the side stream
+        jag, rev = func_token_merge_2d(tokens, S, 3, 3, H, W, mask)
+        back = func_token_split(jag, rev, (1, B, S + H * W, C))
+        qkv = jag.tokens[0, :, :192].reshape(-1, 3, 1, 64).contiguous()
+        cu = jag.offset.to(torch.int32)
+        out = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, S + H * W, perkey_bias=jag.weight.log().bfloat16())
+    side.synchronize()
+    assert torch.equal(rev.cpu(), ref_rev) and torch.equal(jag.offset.cpu(), ref.offset)
+    _assert_features(jag.tokens, ref.tokens, torch.bfloat16)
+    assert torch.equal(back.cpu().reshape(-1, C), jag.tokens[0].cpu()[ref_rev])
+    ref_out, _ = oracle.biased_varlen_attention(qkv.cpu(), cu.cpu(), jag.weight.log().bfloat16().cpu())
+    diff = (out.float().cpu() - ref_out).abs()
+    assert float(diff.max()) <= 1e-2
