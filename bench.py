@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "copy", "e2e", "stress", "stress_e2e", "frame"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "copy", "e2e", "stress", "stress_e2e", "frame"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -278,6 +278,45 @@ def bench_merge_caller_dtypes(device, iters=200, warmup=20):
                      "unmerge_us": round(s_ms / iters * 1e3, 2), "unmerge_bytes": w["split_bytes"],
                      "unmerge_GBs": round(w["split_bytes"] / (s_ms / iters * 1e-3) / 1e9, 1)}
         del w
+        torch.cuda.empty_cache()
+    return out
+
+
+def bench_reference_merge_shapes(device):
+    """The shapes of the reference's own merge / split microbenchmark (test/benchmark/bench_token_merge.py:18-23:
+    1-D groups of 4, fp32 tokens, random mask at 0.5), timed as that script times them: the whole Python call
+    (``func_token_merge`` including its read of the packed row count, ``func_token_split``), synchronised, median."""
+    import torch
+    from come_amd.token_merger import func_token_merge, func_token_split
+
+    def median_ms(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3)
+        return sorted(times)[len(times) // 2]
+
+    out = {}
+    for label, B, M, G, S, C in (("Small", 1, 256, 4, 0, 512), ("Medium", 32, 1024, 4, 2, 1024),
+                                 ("Large", 128, 2048, 4, 2, 2048)):
+        N = S + M * G
+        torch.manual_seed(0)
+        tokens = torch.randn(B, N, C, device=device)
+        mask = torch.rand(B, M, device=device) < 0.5
+        jag, rev = func_token_merge(tokens, S, G, mask)
+        P = jag.tokens.shape[1]
+        reps = 200 if label == "Small" else (50 if label == "Medium" else 10)
+        m_ms = median_ms(lambda: func_token_merge(tokens, S, G, mask), reps)
+        s_ms = median_ms(lambda: func_token_split(jag, rev, (1, B, N, C)), reps)
+        nbytes = (B * N + P) * C * 4
+        out[label] = {"shape": "B=%d N=%d C=%d G=%d fp32, P=%d" % (B, N, C, G, P), "merge_ms": round(m_ms, 4),
+                      "merge_GBs": round(nbytes / (m_ms * 1e-3) / 1e9, 1), "split_ms": round(s_ms, 4),
+                      "split_GBs": round(nbytes / (s_ms * 1e-3) / 1e9, 1)}
+        del tokens, jag, rev
         torch.cuda.empty_cache()
     return out
 
@@ -588,6 +627,8 @@ def main():
             w, wall, ev_ms = bench_attention(args.steps, args.warmup, device)
             print(json.dumps({"only": "attn", "ms_per_call": ev_ms / args.steps,
                               "tflops": w["flops"] / (ev_ms / args.steps * 1e-3) / 1e12}))
+        elif args.only == "refmerge":
+            print(json.dumps({"only": "refmerge", **bench_reference_merge_shapes(device)}))
         elif args.only == "bias":
             print(json.dumps({"only": "bias", **bench_bias_overhead(device)}))
         elif args.only == "dtypes":
@@ -642,6 +683,7 @@ def main():
         other["library_gemm_reference"] = bench_gemm_reference(device)
         other["merge_other_ratios"] = bench_merge_ratios(device)
         other["merge_caller_dtypes"] = bench_merge_caller_dtypes(device)
+        other["reference_merge_microbench_shapes"] = bench_reference_merge_shapes(device)
         other["frame_attention"] = bench_frame_attention(device, w)
         other["bias_overhead"] = bench_bias_overhead(device)
         other["stress"] = bench_stress(device)
