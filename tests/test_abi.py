@@ -80,3 +80,46 @@ def test_header_is_plain_c_and_links_against_the_library(tmp_path):
     run = subprocess.run([str(exe)], capture_output=True, text=True)
     assert run.returncode == 0, run.stderr
     assert run.stdout.startswith(str(_lib.load().come_version()))
+
+
+def test_every_entry_point_rejects_bad_arguments_on_the_host():
+    """Argument checks run before any HIP call, so they can be exercised without a GPU: every entry point
+    returns a non-zero status and leaves a message that names the problem."""
+    lib = _lib.load()
+    BF16, F32 = _lib.COME_BF16, _lib.COME_F32
+
+    def rejected(status, fragment):
+        assert status != 0
+        assert fragment.encode() in lib.come_last_error(), lib.come_last_error()
+
+    rejected(lib.come_token_split(None, 9, 1, 8, None, None, 4, None, None), "dtype")
+    rejected(lib.come_token_split(None, BF16, 1, 0, None, None, 4, None, None), "chans")
+    rejected(lib.come_token_split(None, BF16, 1, 8, None, None, 4, None, None), "rev")            # no index given
+    rejected(lib.come_token_split_pair(None, None, 9, 1, 8, None, None, 4, None, None), "dtype")
+    rejected(lib.come_select_windows(None, _lib.COME_F16, 1, 1, 6, 6, 3, 3, 0, 0.5, None, None, None, 0, None),
+             "come_select_windows")                                                                # fp16 confidence
+    rejected(lib.come_select_windows(None, F32, 1, 1, 6, 6, 0, 3, 0, 0.5, None, None, None, 0, None), "group")
+    rejected(lib.come_select_windows(None, F32, 1, 1, 6, 6, 3, 3, 7, 0.5, None, None, None, 0, None), "mode")
+    rejected(lib.come_select_windows(None, F32, 1, 1, 6, 6, 3, 3, 0, 1.5, None, None, None, 0, None), "threshold")
+    rejected(lib.come_attn_varlen_fwd(None, None, None, F32, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 64,
+                                      None, 10, 0.125, None, 64, 64, None, None), "fp16 and bf16")
+    rejected(lib.come_attn_varlen_fwd(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 0, 10, 1, 64,
+                                      None, 10, 0.125, None, 64, 64, None, None), "batch size")
+    rejected(lib.come_attn_varlen_fwd(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 64,
+                                      None, 10, -1.0, None, 64, 64, None, None), "softmax_scale")
+    rejected(lib.come_attn_varlen_fwd(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 64,
+                                      None, 10, 0.125, None, 64, 64, None, None), "NULL")
+    rejected(lib.come_attn_varlen_fwd_ws(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 32,
+                                         None, 10, 0.125, None, 64, 64, None, None, 0, None), "head_dim")
+    rejected(lib.come_qk_norm_rope(None, None, F32, 64, 64, 64, 64, 4, 1, 64, 1, None, None, None, None, 1e-5,
+                                   None, None, None, 0, None), "bf16 or fp16")
+    rejected(lib.come_qk_norm_rope(None, None, BF16, 64, 64, 64, 64, 4, 1, 32, 1, None, None, None, None, 1e-5,
+                                   None, None, None, 0, None), "head_dim")
+    rejected(lib.come_qk_norm_rope(None, None, BF16, 64, 64, 64, 64, 4, 1, 64, 1, None, None, None, None, 1e-5,
+                                   None, None, None, 0, None), "null")
+    rejected(lib.come_jagged_add_suffix(None, None, 9, 4, 8, None, 2, None, 1, None, None, None, None), "dtype")
+    rejected(lib.come_jagged_add_suffix(None, None, BF16, 4, 8, None, 2, None, 1, None, None, None, None), "offsets")
+    rejected(lib.come_jagged_split_suffix(None, None, BF16, 1, 8, None, 2, 1, None, None, None, None, None), "come_jagged_split_suffix")
+    # sizes that need no work return success without touching the device
+    assert lib.come_token_split(None, BF16, 0, 8, None, None, 0, None, None) == 0
+    assert lib.come_attn_work_bytes(0, 0, 0, 0) == 0
