@@ -340,7 +340,7 @@ __global__ __launch_bounds__(kThreads) void merge_elem_kernel(const MergeArgs a)
 // ---------------------------------------------------------------------------------
 // unmerge: out[i, :] = merged[rev[i], :]
 // ---------------------------------------------------------------------------------
-constexpr int kSplitRows = 1;         // output rows per thread (measured best of 1, 2, 3, 4, 8)
+constexpr int kSplitRows = 1;         // output rows per thread (measured best of 1, 2, 3, 4, 8; the host assumes 1)
 constexpr int kSplitRunRows = 256;    // output rows that stay on one XCD (64 - 1024 measured: no difference)
 
 // PAIR: two packed sources with one index map; an output row holds the row of `merged` followed by the row of
@@ -511,32 +511,51 @@ extern "C" int come_token_merge(const void *tokens, int dtype, int64_t rows, int
     const int64_t row_bytes = chans * dtype_bytes(dtype);
     const bool vec = (row_bytes % 16 == 0) && aligned16(tokens) && aligned16(out);
     a.chunks = static_cast<int>(vec ? row_bytes / 16 : chans);
-    a.group_items = rows * g.groups * a.chunks;
     const int threads = vec ? kMergeThreads : kThreads;
-    a.group_blocks = ceil_div(a.group_items, threads);
-    a.single_items = rows * (g.start + g.tail) * a.chunks;
-    COME_REQUIRE(!vec || (a.group_items < (1ll << 31) && a.single_items < (1ll << 31)), COME_ERR_UNSUPPORTED,
-                 "come_token_merge: more than 2^31 16-byte items in one launch");
     a.by_chunks = make_fastdiv(a.chunks);
     a.by_groups = make_fastdiv(g.groups > 0 ? g.groups : 1);
     a.by_mw = make_fastdiv(g.mw > 0 ? g.mw : 1);
     a.by_per_row = make_fastdiv(g.start + g.tail > 0 ? g.start + g.tail : 1);
     a.by_side = make_fastdiv(g.W - g.cov_w > 0 ? g.W - g.cov_w : 1);
-    const int64_t blocks = a.group_blocks + ceil_div(a.single_items, threads);
-    COME_REQUIRE(blocks < (1ll << 31), COME_ERR_UNSUPPORTED, "come_token_merge: problem too large for one launch");
-    if (blocks == 0) return COME_OK;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (vec) {
-        if (dtype == COME_BF16) launch_merge_vec<COME_BF16>(a, blocks, s);
-        else if (dtype == COME_F16) launch_merge_vec<COME_F16>(a, blocks, s);
-        else launch_merge_vec<COME_F32>(a, blocks, s);
-    } else {
-        const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
-        if (dtype == COME_BF16) hipLaunchKernelGGL(merge_elem_kernel<COME_BF16>, grid, block, 0, s, a);
-        else if (dtype == COME_F16) hipLaunchKernelGGL(merge_elem_kernel<COME_F16>, grid, block, 0, s, a);
-        else hipLaunchKernelGGL(merge_elem_kernel<COME_F32>, grid, block, 0, s, a);
+    // a launch of the 16-byte kernel covers fewer than 2^31 (unit, chunk) items of either kind; more rows take
+    // several launches over consecutive row ranges (packed positions are absolute, so `out` stays where it is)
+    const int64_t per_row_items = static_cast<int64_t>(g.groups > g.start + g.tail ? g.groups : g.start + g.tail) * a.chunks;
+    int64_t rows_per_launch = rows;
+    if (vec && per_row_items > 0) {
+        rows_per_launch = ((1ll << 31) - 1) / per_row_items;
+        COME_REQUIRE(rows_per_launch >= 1, COME_ERR_UNSUPPORTED,
+                     "come_token_merge: more than 2^31 16-byte items in one row");
+        if (rows_per_launch > rows) rows_per_launch = rows;
     }
-    COME_CHECK_LAUNCH("come_token_merge");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t tok_bytes = n_tok * row_bytes;
+    for (int64_t f0 = 0; f0 < rows; f0 += rows_per_launch) {
+        const int64_t nf = rows - f0 < rows_per_launch ? rows - f0 : rows_per_launch;
+        g.rows = static_cast<int>(nf);
+        a.tokens = static_cast<const char *>(tokens) + f0 * tok_bytes;
+        a.mask = merge_mask ? merge_mask + f0 * g.groups : nullptr;
+        a.offsets = offsets + f0;
+        a.prefix = group_prefix ? group_prefix + f0 * g.groups : nullptr;
+        a.rev64 = rev_i64 ? rev_i64 + f0 * n_tok : nullptr;
+        a.rev32 = rev_i32 ? rev_i32 + f0 * n_tok : nullptr;
+        a.group_items = nf * g.groups * a.chunks;
+        a.group_blocks = ceil_div(a.group_items, threads);
+        a.single_items = nf * (g.start + g.tail) * a.chunks;
+        const int64_t blocks = a.group_blocks + ceil_div(a.single_items, threads);
+        COME_REQUIRE(blocks < (1ll << 31), COME_ERR_UNSUPPORTED, "come_token_merge: problem too large for one launch");
+        if (blocks == 0) continue;
+        if (vec) {
+            if (dtype == COME_BF16) launch_merge_vec<COME_BF16>(a, blocks, s);
+            else if (dtype == COME_F16) launch_merge_vec<COME_F16>(a, blocks, s);
+            else launch_merge_vec<COME_F32>(a, blocks, s);
+        } else {
+            const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+            if (dtype == COME_BF16) hipLaunchKernelGGL(merge_elem_kernel<COME_BF16>, grid, block, 0, s, a);
+            else if (dtype == COME_F16) hipLaunchKernelGGL(merge_elem_kernel<COME_F16>, grid, block, 0, s, a);
+            else hipLaunchKernelGGL(merge_elem_kernel<COME_F32>, grid, block, 0, s, a);
+        }
+        COME_CHECK_LAUNCH("come_token_merge");
+    }
     return COME_OK;
 }
 
@@ -558,22 +577,29 @@ static int token_split_impl(const char *who, bool pair, const void *merged, cons
     if (vec) {
         const int chunks = static_cast<int>(row_bytes / 16);
         const int out_chunks = pair ? 2 * chunks : chunks;
-        const int64_t items = ceil_div(total, kSplitRows) * out_chunks;
-        const int64_t blocks = ceil_div(items, kThreads);
-        COME_REQUIRE(items < (1ll << 31), COME_ERR_UNSUPPORTED, "%s: problem too large for one launch", who);
-        const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
+        COME_REQUIRE(out_chunks < (1 << 23), COME_ERR_UNSUPPORTED, "%s: rows wider than 128 MiB are not supported", who);
         const FastDiv by_out_chunks = make_fastdiv(out_chunks);
         const int64_t run64 = static_cast<int64_t>(kSplitRunRows) * out_chunks / kThreads;
         const uint32_t run = static_cast<uint32_t>(run64 < 1 ? 1 : (run64 > 4096 ? 4096 : run64));
-        const uint4 *a4 = static_cast<const uint4 *>(merged), *b4 = static_cast<const uint4 *>(merged_b);
-        uint4 *o4 = static_cast<uint4 *>(out);
+        // a launch covers fewer than 2^31 (row, 16-byte chunk) items; larger outputs take several launches over
+        // consecutive row ranges (whole XCD runs each)
+        int64_t rows_per_launch = ((1ll << 31) - 1) / out_chunks;
+        if (rows_per_launch > kSplitRunRows) rows_per_launch -= rows_per_launch % kSplitRunRows;
+        for (int64_t r0 = 0; r0 < total; r0 += rows_per_launch) {
+            const int64_t nr = total - r0 < rows_per_launch ? total - r0 : rows_per_launch;
+            const int64_t items = nr * out_chunks;
+            const dim3 grid(static_cast<unsigned>(ceil_div(items, kThreads))), block(kThreads);
+            const uint4 *a4 = static_cast<const uint4 *>(merged), *b4 = static_cast<const uint4 *>(merged_b);
+            uint4 *o4 = static_cast<uint4 *>(out) + r0 * out_chunks;
 #define COME_SPLIT_CASE(IDX_, PAIR_, REV_)                                                                       \
-    hipLaunchKernelGGL((split_vec_kernel<IDX_, PAIR_>), grid, block, 0, s, a4, b4, merged_rows, REV_, total,     \
+    hipLaunchKernelGGL((split_vec_kernel<IDX_, PAIR_>), grid, block, 0, s, a4, b4, merged_rows, REV_ + r0, nr,   \
                        chunks, o4, items, by_out_chunks, run)
-        if (rev_i64 && pair) COME_SPLIT_CASE(int64_t, true, rev_i64);
-        else if (rev_i64) COME_SPLIT_CASE(int64_t, false, rev_i64);
-        else if (pair) COME_SPLIT_CASE(int32_t, true, rev_i32);
-        else COME_SPLIT_CASE(int32_t, false, rev_i32);
+            if (rev_i64 && pair) COME_SPLIT_CASE(int64_t, true, rev_i64);
+            else if (rev_i64) COME_SPLIT_CASE(int64_t, false, rev_i64);
+            else if (pair) COME_SPLIT_CASE(int32_t, true, rev_i32);
+            else COME_SPLIT_CASE(int32_t, false, rev_i32);
+            COME_CHECK_LAUNCH(who);
+        }
 #undef COME_SPLIT_CASE
     } else {
         const int eb = dtype_bytes(dtype);

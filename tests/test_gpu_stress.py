@@ -8,7 +8,7 @@ import torch
 
 import oracle
 from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
-from come_amd.token_merger import func_token_merge_2d, func_token_split
+from come_amd.token_merger import func_token_merge, func_token_merge_2d, func_token_split
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -114,3 +114,64 @@ def test_unmerged_global_segment_of_133k_tokens_sampled():
         diff = (out[row] - ref).abs()
         assert float(diff.max()) <= 1e-2 and float(diff.mean()) <= 1e-3
         torch.testing.assert_close(lse[:, row], torch.logsumexp(scores, -1), atol=2e-3, rtol=1e-3)
+
+
+def _needs_free_memory(gib):
+    free, _ = torch.cuda.mem_get_info()
+    if free < gib * (1 << 30):
+        pytest.skip(f"needs {gib} GiB of free device memory")
+
+
+def test_unmerge_beyond_one_launch():
+    """More than 2^31 (row, 16-byte chunk) items: the entry point covers the output with several launches over
+    consecutive row ranges.  2.2 M rows of 16 KiB (36 GB) gathered from 1000 packed rows; rows around the launch
+    border and at both ends are compared with the gather they stand for."""
+    _needs_free_memory(60)
+    from come_amd.cuda_extension import co_me_cuext
+    C, P, total = 8192, 1000, 2_200_000
+    assert total * (C * 2 // 16) > 2 ** 31
+    g = torch.Generator(device=DEV).manual_seed(0)
+    merged = torch.randn(P, C, device=DEV, generator=g).bfloat16()
+    rev = torch.randint(0, P, (total,), device=DEV, generator=g, dtype=torch.int32)
+    out = co_me_cuext.co_me_token_split_cuda(merged, rev, C)
+    assert out.shape == (total, C)
+    border = ((2 ** 31 - 1) // (C * 2 // 16)) // 256 * 256                      # first row of the second launch
+    rows = torch.tensor([0, 1, 255, 256, border - 1, border, border + 1, border + 255, total - 2, total - 1], device=DEV)
+    assert torch.equal(out[rows], merged[rev[rows].long()])
+    step = torch.arange(0, total, 9973, device=DEV)
+    assert torch.equal(out[step], merged[rev[step].long()])
+
+
+def test_merge_beyond_one_launch():
+    """The same for the merge: 4200 rows of 1032 tokens x 8192 channels (71 GB of bf16 tokens, 1-D groups of 2)
+    exceed 2^31 (unit, chunk) items, so the rows are covered by two launches.  Frames at the ends and on both sides
+    of the launch border are compared with the oracle."""
+    _needs_free_memory(160)
+    rows, S, M, G, C = 4200, 8, 512, 2, 8192
+    N = S + M * G
+    per_row_items = max(M, S) * (C * 2 // 16)
+    border = (2 ** 31 - 1) // per_row_items                                          # first row of the second launch
+    assert 0 < border < rows
+    # small integers: every mean of two of them is exact in bf16, so packed rows can be compared bit for bit
+    pattern = (torch.arange(rows * N, device=DEV) % 61).to(torch.bfloat16).view(rows, N, 1)
+    tokens = torch.empty(rows, N, C, dtype=torch.bfloat16, device=DEV)
+    tokens.copy_(pattern)
+    g = torch.Generator(device=DEV).manual_seed(1)
+    mask = torch.rand(rows, M, device=DEV, generator=g) < 0.5
+    jag, rev = func_token_merge(tokens, S, G, mask)
+    P = jag.tokens.shape[1]
+    assert P == rows * N - int(mask.sum()) * (G - 1) == int(jag.offset[-1])
+    assert float(jag.weight.sum()) == rows * N
+    for f in (0, border - 1, border, border + 1, rows - 1):
+        ref, ref_rev = oracle.token_merge_1d(tokens[f:f + 1, :, :16].cpu(), S, G, mask[f:f + 1].cpu())
+        lo, hi = int(jag.offset[f]), int(jag.offset[f + 1])
+        assert hi - lo == ref.tokens.shape[1]
+        got = jag.tokens[0, lo:hi]
+        assert torch.equal(got[:, :16].cpu(), ref.tokens[0])
+        assert torch.equal(got[:, -1].cpu(), ref.tokens[0][:, 0])                    # last channel chunk as well
+        assert torch.equal(rev[f * N:(f + 1) * N].cpu() - lo, ref_rev)
+        assert torch.equal(jag.weight[lo:hi].cpu(), ref.weight)
+    del tokens
+    back = func_token_split(jag, rev, (1, rows, N, C))
+    idx = torch.tensor([0, N - 1, border * N - 1, border * N, rows * N - 1], device=DEV)
+    assert torch.equal(back.view(-1, C)[idx], jag.tokens[0][rev[idx]])
