@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "copy", "e2e", "stress", "stress_e2e", "frame"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "power", "copy", "e2e", "stress", "stress_e2e", "frame"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -424,6 +424,79 @@ def bench_bias_overhead(device):
     return out
 
 
+def bench_power(device, seconds=4.0):
+    """Board power (hwmon ``power1_input`` / ``power1_average`` of the GPU, sampled every 20 ms from sysfs) while
+    the headline attention launch and the library bf16 GEMM run back to back for ``seconds`` each, on N(0,1) and on
+    all-zero operands.  Shows which of the two limits a kernel runs into: its own schedule or the power cap."""
+    import glob
+    import threading
+
+    import torch
+    from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
+
+    files = {}
+    for name in ("power1_average", "power1_input", "power1_cap"):
+        files[name] = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/" + name))
+
+    def read(name):
+        vals = []
+        for f in files.get(name, []):
+            try:
+                with open(f) as fh:
+                    vals.append(int(fh.read().strip()))
+            except (OSError, ValueError):
+                pass
+        return vals
+
+    def watts():
+        vals = read("power1_average") or read("power1_input")
+        return max(vals) / 1e6 if vals else None
+
+    def phase(fn, flops):
+        samples, stop = [], threading.Event()
+
+        def sampler():
+            while not stop.is_set():
+                samples.append(watts())
+                time.sleep(0.02)
+
+        t = threading.Thread(target=sampler)
+        t.start()
+        t0, calls = time.perf_counter(), 0
+        while time.perf_counter() - t0 < seconds:
+            if fn is None:
+                time.sleep(0.05)
+            else:
+                for _ in range(10):
+                    fn()
+                torch.cuda.synchronize()
+                calls += 10
+        dt = time.perf_counter() - t0
+        stop.set()
+        t.join()
+        steady = [x for x in samples[len(samples) // 3:] if x is not None]
+        out = {"power_W": round(sum(steady) / len(steady), 1) if steady else None}
+        if calls:
+            out.update(ms_per_call=round(dt / calls * 1e3, 3), TFLOPs=round(flops * calls / dt / 1e12, 1))
+        return out
+
+    w = make_attention_workload(device)
+    zeros = torch.zeros_like(w["qkv"])
+    max_len = max(w["lens"])
+    a = torch.randn(8192, 8192, device=device).bfloat16()
+    b = torch.randn(8192, 8192, device=device).bfloat16()
+    z = torch.zeros_like(a)
+    cap = read("power1_cap")
+
+    def attn(qkv):
+        return lambda: flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, w["cu"], max_len, perkey_bias=w["bias"],
+                                                                      softmax_scale=0.125)
+
+    return {"power_cap_W": max(cap) / 1e6 if cap else None, "idle": phase(None, 0),
+            "attention_normal": phase(attn(w["qkv"]), w["flops"]), "attention_zeros": phase(attn(zeros), w["flops"]),
+            "gemm_8192_normal": phase(lambda: a @ b, 2.0 * 8192 ** 3), "gemm_8192_zeros": phase(lambda: z @ z, 2.0 * 8192 ** 3)}
+
+
 def bench_frame_attention(device, w):
     """Frame-mode attention of the headline workload's first sequence: 32 segments of about 798 tokens."""
     import torch
@@ -627,6 +700,8 @@ def main():
             w, wall, ev_ms = bench_attention(args.steps, args.warmup, device)
             print(json.dumps({"only": "attn", "ms_per_call": ev_ms / args.steps,
                               "tflops": w["flops"] / (ev_ms / args.steps * 1e-3) / 1e12}))
+        elif args.only == "power":                               # 20 s of sustained load: not part of the default run
+            print(json.dumps({"only": "power", **bench_power(device)}))
         elif args.only == "refmerge":
             print(json.dumps({"only": "refmerge", **bench_reference_merge_shapes(device)}))
         elif args.only == "bias":
