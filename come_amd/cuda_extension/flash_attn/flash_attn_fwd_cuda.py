@@ -3,7 +3,7 @@
 Positional signatures and return lists follow the reference's pybind module
 ``flash_attn_fwd_cuda`` (``src/cuda_extension/flash_attn/flash_api.cpp:538-607``,
 checks ``:291-408``, bias checks ``:274-288``).  Only what the Co-Me call sites
-reach is implemented: fp16 / bf16, head_dim 64, self-attention over one set of
+reach is implemented: fp16 / bf16, head_dim 64 (narrower heads are zero-padded to it), self-attention over one set of
 ``cu_seqlens``, no causal mask, no dropout, no alibi / softcap / sliding window /
 paged KV / left padding.  Anything else raises ``RuntimeError`` instead of
 computing something different.
@@ -101,8 +101,8 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
     _check(tuple(v.shape) == (total_k, num_heads_k, head_size), "v must have shape (total_k, num_heads_k, head_size)")
     _check(tuple(cu_seqlens_k.shape) == (batch_size + 1,), "cu_seqlens_k must have shape (batch_size + 1)")
     _unsupported(num_heads != num_heads_k, "grouped-query attention (num_heads != num_heads_k)")
-    if head_size != 64:
-        _unsupported(True, f"head_dim {head_size} (only 64 is implemented)")
+    if head_size > 64:
+        _unsupported(True, f"head_dim {head_size} (64 and, zero-padded, smaller multiples of 8 are implemented)")
     _unsupported(total_q != total_k or max_seqlen_q != max_seqlen_k
                  or (cu_seqlens_q.data_ptr() != cu_seqlens_k.data_ptr() and not torch.equal(cu_seqlens_q, cu_seqlens_k)),
                  "cross attention (different query and key packing)")
@@ -118,6 +118,24 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
 
     def _aligned(t):          # the kernel issues 16-byte loads
         return t.data_ptr() % 16 == 0 and t.stride(0) % 8 == 0 and t.stride(1) % 8 == 0
+
+    if head_size < 64:
+        # narrower heads run on the 64-wide kernel: zero columns change neither q . k nor the other columns of
+        # the output (softmax_scale was fixed by the caller from the real width); costs a padded copy of q, k, v
+        padded = _varlen_fwd_impl(*(torch.nn.functional.pad(t, [0, 64 - head_size]) for t in (q, k, v)), None,
+                                  cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
+                                  perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, False, is_causal,
+                                  window_size_left, window_size_right, softcap, return_softmax, gen)
+        narrow = padded[0][..., :head_size]
+        if out_ is not None:
+            _check(out_.dtype == q.dtype and tuple(out_.shape) == (total_q, num_heads, head_size),
+                   "out has the wrong shape or dtype")
+            out_.copy_(narrow)
+            narrow = out_
+        else:
+            narrow = narrow.contiguous()
+        return [narrow, padded[1], padded[2], padded[3]]
+
     q, k, v = (t if _aligned(t) else t.contiguous() for t in (q, k, v))
 
     with _on_device(dev):
