@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "power", "copy", "e2e", "stress", "stress_e2e", "frame"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "power", "prologue", "copy", "e2e", "stress", "stress_e2e", "frame"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -497,6 +497,43 @@ def bench_power(device, seconds=4.0):
             "gemm_8192_normal": phase(lambda: a @ b, 2.0 * 8192 ** 3), "gemm_8192_zeros": phase(lambda: z @ z, 2.0 * 8192 ** 3)}
 
 
+def bench_qk_prologue(device, rows=(25536, 43968), iters=200, warmup=20):
+    """q / k LayerNorm + 2-D RoPE in place on the packed ``qkv [P, 3, 16, 64]`` bf16 (one launch through the C ABI),
+    over 4 rotating tensors (each launch touches 2/3 of 157 MB at P = 25 536).  Algorithmic bytes: q and k read and
+    written once."""
+    import torch
+    from come_amd import _lib
+    from come_amd.common import RotaryPositionEmbedding2D
+
+    lib, stream = _lib.load(), _lib.current_stream(device)
+    out = {}
+    for P in rows:
+        H = 16
+        torch.manual_seed(3)
+        sets = [torch.randn(P, 3, H, 64, device=device).bfloat16() for _ in range(4)]
+        params = [torch.randn(64, device=device).bfloat16() for _ in range(4)]
+        cos_t, sin_t = RotaryPositionEmbedding2D(100.0).tables(64, 38, device, torch.bfloat16)
+        pos = torch.randint(0, 38, (P, 2), device=device)
+        state = {"i": 0}
+
+        def step():
+            i = state["i"] = (state["i"] + 1) % 4
+            q, k = sets[i][:, 0], sets[i][:, 1]
+            _lib.check(lib.come_qk_norm_rope(q.data_ptr(), k.data_ptr(), _lib.COME_BF16, q.stride(0), q.stride(1),
+                                             k.stride(0), k.stride(1), P, H, 64, 1, params[0].data_ptr(),
+                                             params[1].data_ptr(), params[2].data_ptr(), params[3].data_ptr(), 1e-5,
+                                             pos.data_ptr(), cos_t.data_ptr(), sin_t.data_ptr(), 38, stream))
+
+        _, ms = time_loop(step, iters, warmup)
+        nbytes = P * 2 * H * 64 * 2 * 2
+        gbs = nbytes / (ms / iters * 1e-3) / 1e9
+        out["P=%d" % P] = {"us_per_call": round(ms / iters * 1e3, 2), "algorithmic_bytes": nbytes, "GBs": round(gbs, 1),
+                           "frac": round(gbs / PEAK_HBM_GBS, 4)}
+        del sets
+        torch.cuda.empty_cache()
+    return out
+
+
 def bench_frame_attention(device, w):
     """Frame-mode attention of the headline workload's first sequence: 32 segments of about 798 tokens."""
     import torch
@@ -702,6 +739,8 @@ def main():
                               "tflops": w["flops"] / (ev_ms / args.steps * 1e-3) / 1e12}))
         elif args.only == "power":                               # 20 s of sustained load: not part of the default run
             print(json.dumps({"only": "power", **bench_power(device)}))
+        elif args.only == "prologue":
+            print(json.dumps({"only": "prologue", **bench_qk_prologue(device, iters=args.steps, warmup=args.warmup)}))
         elif args.only == "refmerge":
             print(json.dumps({"only": "refmerge", **bench_reference_merge_shapes(device)}))
         elif args.only == "bias":
@@ -759,6 +798,7 @@ def main():
         other["merge_other_ratios"] = bench_merge_ratios(device)
         other["merge_caller_dtypes"] = bench_merge_caller_dtypes(device)
         other["reference_merge_microbench_shapes"] = bench_reference_merge_shapes(device)
+        other["qk_prologue"] = bench_qk_prologue(device)
         other["frame_attention"] = bench_frame_attention(device, w)
         other["bias_overhead"] = bench_bias_overhead(device)
         other["stress"] = bench_stress(device)
