@@ -229,7 +229,7 @@ def merge_workload(device, ratio=0.5, sets=None, frames=16, H=37, W=37, jitter=N
     merge_bytes = (frames * N * C * esize + P * C * esize + frames * N * 4 + P * 4 + frames * H * W * 4
                    + (frames + 1) * 4)
     split_bytes = P * C * esize + frames * N * 4 + frames * N * C * esize
-    return dict(merge_only=merge_only, pipeline=pipeline, split_only=split_only, P=P, merge_bytes=merge_bytes,
+    return dict(merge_only=merge_only, pipeline=pipeline, select_and_plan=select_and_plan, split_only=split_only, P=P, merge_bytes=merge_bytes,
                 split_bytes=split_bytes, frames=frames, N=N, C=C, ratio=ratio, tokens=tokens, conf=conf,
                 counts=counts, offsets=offsets, outs=outs, restored=restored, index_map=index_map,
                 keep=(mask, means, prefix))
@@ -241,6 +241,7 @@ def bench_merge_unmerge(device, iters=200, warmup=20):
         w["merge_only"]()                                       # fill every output set before unmerge reads it
     _, merge_ms = time_loop(w["merge_only"], iters, warmup)
     _, pipe_ms = time_loop(w["pipeline"], iters, warmup)
+    _, select_plan_ms = time_loop(w["select_and_plan"], iters, warmup)
     _, split_ms = time_loop(w["split_only"], iters, warmup)
     merge_gbs = w["merge_bytes"] / (merge_ms / iters * 1e-3) / 1e9
     split_gbs = w["split_bytes"] / (split_ms / iters * 1e-3) / 1e9
@@ -250,7 +251,8 @@ def bench_merge_unmerge(device, iters=200, warmup=20):
                   "algorithmic_bytes": w["merge_bytes"], "iters": iters, "rotating_buffer_sets": len(w["outs"]),
                   "roofline": {"bound": "hbm", "achieved": round(merge_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                "frac": round(merge_gbs / PEAK_HBM_GBS, 4), "traffic": TRAFFIC_BYTES["merge"]},
-                  "select_plan_merge_us": round(pipe_ms / iters * 1e3, 2)},
+                  "select_plan_merge_us": round(pipe_ms / iters * 1e3, 2),
+                  "select_plan_us": round(select_plan_ms / iters * 1e3, 2)},
         "unmerge": {"workload": "C2 unmerge: P=%d -> %d rows, C=1024 bf16" % (w["P"], w["frames"] * w["N"]),
                     "value": round(split_gbs, 1), "unit": "GB/s", "us_per_call": round(split_ms / iters * 1e3, 2),
                     "algorithmic_bytes": w["split_bytes"], "iters": iters, "rotating_buffer_sets": len(w["outs"]),
