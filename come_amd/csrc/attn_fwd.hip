@@ -172,11 +172,11 @@ constexpr int kStages = 4;
 // awaited explicitly with s_waitcnt vmcnt before the barrier that publishes the tile.
 __device__ inline void dma_b128(const char *base, uint32_t lane_offset, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :: "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory");
+                 :: "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory", "m0");
 }
 __device__ inline void dma_b32(const char *base, uint32_t lane_offset, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
-                 :: "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory");
+                 :: "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory", "m0");
 }
 __device__ inline uint32_t lds_address(const void *p) {
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void *)(p)));

@@ -227,12 +227,14 @@ __global__ __launch_bounds__(kSelectThreads) void select_windows_kernel(
 
     // 2. threshold.  Ranking: the two neighbouring order statistics of torch.quantile's linear interpolation;
     //    the upper one is either the same value again (duplicates) or the smallest value above the lower one.
-    float cut = threshold;
+    //    Absolute and normalised score compare a tensor of the confidence dtype with a scalar: the scalar is
+    //    rounded to that dtype first, as the tensor library does (a bf16 mean of 0.44921875 is not below 0.45).
+    float cut = round_dt<DT>(threshold);
     if (mode == 0) {
         const float a = radix_select(my_means, mine, in_regs, n, rank_lo, hist, ctl, reinterpret_cast<uint32_t *>(red));
         float b = a;
         if (rank_hi != rank_lo) {
-            float le = 0.f;                                   // exact in fp32: n < 2^24
+            float le = 0.f;                                   // exact in fp32: n < 2^24 (checked by the host)
             uint32_t above = 0xffffffffu;                     // ordered key of the smallest value > a
             const uint32_t key_a = ordered_key(a);
             auto visit = [&](float x) {
@@ -300,7 +302,8 @@ extern "C" int come_select_windows(const void *conf, int dtype, int64_t batch, i
     const int64_t windows = (grid_h / group_h) * (grid_w / group_w);
     const int64_t n = frames * windows;
     if (batch == 0 || n == 0) return COME_OK;
-    COME_REQUIRE(n < (1ll << 30) && batch < (1ll << 31) && batch * frames * grid_h * grid_w < (1ll << 40),
+    // n < 2^24: ranks and counts of windows are exact in fp32, which is also what the quantile's fp32 rank needs
+    COME_REQUIRE(n < (1ll << 24) && batch < (1ll << 31) && batch * frames * grid_h * grid_w < (1ll << 40),
                  COME_ERR_UNSUPPORTED, "come_select_windows: problem too large");
     COME_REQUIRE(conf && merge_mask, COME_ERR_INVALID, "come_select_windows: conf / merge_mask is NULL");
     float *means = means_f32;

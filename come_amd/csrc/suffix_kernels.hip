@@ -18,7 +18,7 @@ struct SuffixArgs {
     float *out_weight;
     int64_t *out_offsets;         // [n_seg + 1]
     uint8_t *suffix_out;          // strip: [n_seg, T, row_bytes]
-    int64_t rows_out, n_seg, T;
+    int64_t rows_in, rows_out, n_seg, T;
     int64_t row_bytes;
     int unit;                     // bytes moved per thread: 16, 4 or 2
     int units_per_row;
@@ -57,14 +57,17 @@ __global__ __launch_bounds__(kThreads) void suffix_kernel(const SuffixArgs a) {
         const int64_t s = find_segment(a.offsets, a.n_seg, step, row);
         const int64_t j = row - (a.offsets[s] + s * step);               // position inside the output segment
         const int64_t len_in = a.offsets[s + 1] - a.offsets[s];
+        // The offsets come from device memory that the host cannot check: indices derived from them are clamped
+        // into the tensors, so that inconsistent offsets give wrong rows instead of accesses outside them.
         const uint8_t *src;
         float w = 1.f;
-        if (a.strip || j < len_in) {
-            const int64_t r = a.offsets[s] + j;
+        if (a.rows_in > 0 && (a.strip || j < len_in)) {
+            const int64_t r = min(max(a.offsets[s] + j, int64_t{0}), a.rows_in - 1);
             src = a.tokens + r * a.row_bytes;
             if (a.weight) w = a.weight[r];
         } else {
-            src = a.suffix_in + (s * a.T + (j - len_in)) * a.row_bytes;
+            const int64_t t = min(max(j - len_in, int64_t{0}), a.T - 1);
+            src = a.suffix_in + (s * a.T + t) * a.row_bytes;
         }
         copy_unit(a.out_tokens + row * a.row_bytes + col, src + col, a.unit);
         if (col == 0 && a.out_weight) a.out_weight[row] = w;
@@ -72,8 +75,8 @@ __global__ __launch_bounds__(kThreads) void suffix_kernel(const SuffixArgs a) {
         const int64_t e = row - body_rows;                               // (segment, t) of the stripped block
         const int64_t s = e / a.T;
         const int64_t t = e - s * a.T;
-        int64_t r = a.offsets[s + 1] - a.T + t;
-        r = r < 0 ? 0 : r;                                               // a segment shorter than T (caller error) stays in bounds
+        // a segment shorter than T (caller error) or inconsistent offsets stay in bounds
+        const int64_t r = min(max(a.offsets[s + 1] - a.T + t, int64_t{0}), a.rows_in - 1);
         copy_unit(a.suffix_out + e * a.row_bytes + col, a.tokens + r * a.row_bytes + col, a.unit);
     }
 }
@@ -122,6 +125,7 @@ extern "C" int come_jagged_add_suffix(const void *tokens, const float *weight, i
     a.out_tokens = static_cast<uint8_t *>(out_tokens);
     a.out_weight = out_weight;
     a.out_offsets = out_offsets;
+    a.rows_in = rows;
     a.rows_out = rows + n_seg * count;
     a.n_seg = n_seg;
     a.T = count;
@@ -156,6 +160,7 @@ extern "C" int come_jagged_split_suffix(const void *tokens, const float *weight,
     a.out_weight = out_weight;
     a.out_offsets = out_offsets;
     a.suffix_out = static_cast<uint8_t *>(out_suffix);
+    a.rows_in = rows;
     a.rows_out = rows - n_seg * count;
     a.n_seg = n_seg;
     a.T = count;

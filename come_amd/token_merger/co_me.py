@@ -91,10 +91,12 @@ class CoMe_TokenMerger(ITokenMerger):
             confidence = self.predictor(feature.permute(0, 1, 3, 4, 2).bfloat16())
         if self.conf_mode == "pairwise-rank" and not (0.0 <= self.threshold <= 1.0):
             raise ValueError(f"Ranking mode requires threshold in [0, 1], got {self.threshold}")
-        # groups of G consecutive tokens are 1 x G windows of a 1 x (H*W) grid; the ranking is per
-        # frame here (co_me.py:65-73 takes the quantile over the last dimension of [B*S, M])
+        # groups of G consecutive tokens are 1 x G windows of a 1 x (H*W) grid.  Scope of the statistics as in the
+        # reference: the ranking takes its quantile over the last dimension of [B*S, M], i.e. per frame
+        # (co_me.py:65-70), the normalised score is normalised over the whole batch element (co_me.py:54-58)
         conf = confidence.reshape(B * S, 1, H * W)
-        mask = co_me_cuext.co_me_select_windows(conf, B * S, 1, self.group_size, self.threshold, self.conf_mode)
+        batch = B if self.conf_mode == "mse" else B * S
+        mask = co_me_cuext.co_me_select_windows(conf, batch, 1, self.group_size, self.threshold, self.conf_mode)
         return mask, (B, S, C, H, W)
 
     def merge(self, ctx, tokens: torch.Tensor, stub: Any | None = None, *, start_index: int | None = None):

@@ -138,14 +138,16 @@ int come_token_split_pair(const void *merged_a, const void *merged_b, int dtype,
  *   mode     0 = ranking: per batch element, over its frames * windows means jointly,
  *                mask = mean < quantile(float(mean), threshold) with torch.quantile's
  *                linear interpolation;
- *            1 = absolute: mask = mean < threshold
+ *            1 = absolute: mask = mean < threshold (threshold rounded to `dtype` first, as a
+ *                comparison of a `dtype` tensor with a scalar does)
  *            2 = normalised: the confidence of a batch element is first turned into
  *                z = (x - mean) / (std + 1e-3) over all its positions (unbiased std, every
- *                step rounded to `dtype`), then mask = window mean of z < threshold
+ *                step rounded to `dtype`), then mask = window mean of z < threshold (rounded likewise)
  *   means_f32 [batch * frames, windows] float out (the means, rounded to `dtype` first);
  *            may be NULL
  *   merge_mask [batch * frames, windows] bytes out (1 = merge)
- *   work     device scratch of at least come_select_work_bytes(...) bytes
+ *   work     device scratch that holds the means when means_f32 is NULL: at least
+ *            come_select_work_bytes(...) bytes; not used (may be NULL) when means_f32 is given
  *
  * Stands in for the window-mean + torch.quantile + compare sequence of
  * _CoMe_2D_Base.build_ctx (src/accelerate/token_merger/co_me_2d.py:268-298; mode 2:

@@ -28,7 +28,13 @@ Pinning status of each function (what fixes its answers besides this text):
   select_lowest_confidence            tests (nothing there calls build_ctx).
                                       Pinned here by library composition
                                       (torch.quantile), numpy.quantile, a sort
-                                      based closed form and count identities.
+                                      based closed form and count identities;
+                                      the normalised-score branch by a
+                                      hand-computed case and an fp64 loop
+                                      brute force.
+  select_groups_1d                    same status (the 1-D merger's build_ctx);
+                                      same pins plus its per-frame ranking /
+                                      per-batch-element normalisation scope.
   biased_varlen_attention             closed form softmax(q k^T s + b) v used by
                                       the reference's tests; reductions to
                                       torch SDPA, key-duplication identity,
@@ -53,6 +59,7 @@ from .token_merge import (  # noqa: F401
 from .selection import (  # noqa: F401
     window_confidence_means,
     select_lowest_confidence,
+    select_groups_1d,
     quantile_threshold,
 )
 from .attention import (  # noqa: F401

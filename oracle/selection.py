@@ -11,7 +11,13 @@ the very library calls the reference makes (``Tensor.mean``,
 ``torch.quantile``, ``<``); ``quantile_threshold`` is an independent sort-based
 restatement of ``torch.quantile`` checked against it and against
 ``numpy.quantile``; and for distinct values the number of selected windows has
-the closed form ``floor(r (n-1)) + 1`` (``r (n-1)`` not an integer).
+the closed form ``floor(r (n-1)) + 1`` (``r (n-1)`` not an integer).  The
+normalised-score branch is pinned by a hand-computed case (values 0..3: mean
+1.5, unbiased standard deviation sqrt(5/3)) whose thresholds separate it from
+a biased deviation and from a missing ``+ 1e-3``, and by an fp64 loop brute
+force (``tests/bruteforce.py``).  ``select_groups_1d`` restates the 1-D
+merger's ``build_ctx`` (``src/accelerate/token_merger/co_me.py:47-73``) and is
+pinned the same way plus by its per-frame / per-batch-element scope.
 """
 
 from __future__ import annotations
@@ -91,4 +97,41 @@ def select_lowest_confidence(
         flat = conf.reshape(batch, -1)
         z = (flat - flat.mean(dim=-1, keepdim=True)) / (flat.std(dim=-1, keepdim=True) + 1e-3)
         return window_confidence_means(z.reshape(F, H, W), group_h, group_w) < threshold
+    raise ValueError(f"unknown confidence mode {mode!r}")
+
+
+def select_groups_1d(
+    confidence: torch.Tensor,
+    batch: int,
+    frames: int,
+    group_size: int,
+    threshold: float,
+    mode: str = "pairwise-rank",
+) -> torch.Tensor:
+    """1-D merger: ``confidence [B, S*H*W]`` -> ``mask [B*S, H*W // G] bool``.
+
+    Restates ``CoMe_TokenMerger.build_ctx`` (reference
+    ``src/accelerate/token_merger/co_me.py:47-73``).  Scope of each mode there:
+      * ``"mse"``: z-score over the whole batch element (``[B, -1]``, ``:54-58``),
+        then the mean of each group of ``G`` consecutive scores;
+      * ``"pairwise-rank"``: the quantile is taken over the last dimension of
+        ``[B*S, M]``, i.e. per frame (``:65-70``), not jointly as in the 2-D merger;
+      * ``"abs_mse"``: group mean ``< threshold`` (``:72-74``).
+    """
+    per_frame = confidence.numel() // (batch * frames)
+    if per_frame % group_size != 0:
+        raise ValueError(f"H * W ({per_frame}) must be divisible by group_size ({group_size})")
+    groups = per_frame // group_size
+    if mode == "mse":
+        flat = confidence.reshape(batch, -1)
+        z = (flat - flat.mean(dim=-1, keepdim=True)) / (flat.std(dim=-1, keepdim=True) + 1e-3)
+        return z.reshape(batch * frames, groups, group_size).mean(dim=-1) < threshold
+    means = confidence.reshape(batch * frames, groups, group_size).mean(dim=-1)
+    if mode == "pairwise-rank":
+        if not (0.0 <= threshold <= 1.0):
+            raise ValueError(f"Ranking mode requires threshold in [0, 1], got {threshold}")
+        cut = torch.quantile(means.float(), threshold, dim=-1, keepdim=True)
+        return means < cut
+    if mode == "abs_mse":
+        return means < threshold
     raise ValueError(f"unknown confidence mode {mode!r}")

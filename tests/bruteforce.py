@@ -78,3 +78,31 @@ def attention_loops(q, k, v, bias, scale):
         for j in range(L):
             out[i] += (e[j] / z) * v[j]
     return out, lse
+
+
+def zscore_window_means_loops(conf, batch, gh, gw):
+    """Normalised-score window means by plain loops in float64.
+
+    conf: np [batch * frames, H, W].  Per batch element: mean over all of its positions, standard
+    deviation with the n - 1 divisor, z = (x - mean) / (std + 1e-3); then the mean of z over every
+    full gh x gw window (block-row-major).  Returns np [batch * frames, M].
+    """
+    F, H, W = conf.shape
+    frames = F // batch
+    mh, mw = H // gh, W // gw
+    out = np.zeros((F, mh * mw))
+    for b in range(batch):
+        vals = [float(conf[b * frames + f, y, x]) for f in range(frames) for y in range(H) for x in range(W)]
+        n = len(vals)
+        mean = sum(vals) / n
+        var = sum((v - mean) * (v - mean) for v in vals) / (n - 1)
+        denom = math.sqrt(var) + 1e-3
+        for f in range(frames):
+            for wy in range(mh):
+                for wx in range(mw):
+                    acc = 0.0
+                    for dy in range(gh):
+                        for dx in range(gw):
+                            acc += (float(conf[b * frames + f, wy * gh + dy, wx * gw + dx]) - mean) / denom
+                    out[b * frames + f, wy * mw + wx] = acc / (gh * gw)
+    return out

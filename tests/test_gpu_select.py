@@ -76,6 +76,21 @@ def test_negative_values_and_absolute_mode():
     assert torch.equal(mask.cpu(), oracle.select_lowest_confidence(conf, 1, 3, 3, 0.1, mode="abs_mse"))
 
 
+def test_scalar_threshold_is_rounded_to_the_confidence_dtype():
+    """`bf16 tensor < 0.45` compares against bf16(0.45) = 0.44921875: a window whose mean is exactly that value is
+    not selected, although it is below 0.45 (reference co_me_2d.py:297-298 with a bf16 predictor output)."""
+    conf = torch.full((2, 6, 6), 0.44921875).bfloat16()
+    conf[1, :3, :3] = 0.4453125                                   # one step further down: selected
+    for mode in ("abs_mse",):
+        mask = co_me_cuext.co_me_select_windows(conf.to(DEV), 1, 3, 3, 0.45, mode=mode)
+        want = oracle.select_lowest_confidence(conf, 1, 3, 3, 0.45, mode=mode)
+        assert want.reshape(-1).tolist() == [False] * 4 + [True] + [False] * 3
+        assert torch.equal(mask.cpu(), want)
+    # fp32 confidence keeps the fp32 threshold
+    mask = co_me_cuext.co_me_select_windows(conf.float().to(DEV), 1, 3, 3, 0.45, mode="abs_mse")
+    assert bool(mask.all())
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("batch,frames,H,W", [(1, 4, 12, 12), (2, 8, 37, 37), (1, 32, 37, 28)])
 def test_normalised_score_mode(batch, frames, H, W, dtype):
@@ -98,6 +113,45 @@ def test_normalised_score_mode(batch, frames, H, W, dtype):
     assert float(clear.float().mean()) > 0.9
     assert torch.equal(mask.cpu()[clear], want[clear])
     assert 0 < int(mask.sum()) < mask.numel()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_normalised_score_hand_computed_case(dtype):
+    """Values 0, 1, 2, 3: mean 1.5, unbiased standard deviation sqrt(5 / 3) = 1.2909944, so
+    z = (-1.5, -0.5, 0.5, 1.5) / 1.2919944 = (-1.1610, -0.3870, 0.3870, 1.1610) (bf16 rounds the denominator to
+    1.2890625 and z to -1.1640625 ...).  The thresholds separate that from a biased deviation (z0 = -1.34) in
+    both dtypes and, in fp32, from a missing + 1e-3 (z0 = -1.16190 instead of -1.16100)."""
+    conf = torch.tensor([[[0.0, 1.0], [2.0, 3.0]]]).to(dtype)
+    z = [-1.1609958, -0.3869986, 0.3869986, 1.1609958]
+    thresholds = [-1.5, -1.25, -1.0, -0.5, -0.3, 0.0, 0.4, 1.0, 1.25]
+    if dtype == torch.float32:
+        thresholds += [-1.1615, -1.1605]
+    for thr in thresholds:
+        mask, means = co_me_cuext.co_me_select_windows(conf.to(DEV), 1, 1, 1, thr, mode="mse", return_means=True)
+        assert mask.cpu().reshape(-1).tolist() == [v < thr for v in z], thr
+        assert torch.equal(mask.cpu(), oracle.select_lowest_confidence(conf, 1, 1, 1, thr, mode="mse"))
+        torch.testing.assert_close(means.cpu().reshape(-1), torch.tensor(z),
+                                   atol=2.0 ** -8 if dtype == torch.bfloat16 else 2e-7, rtol=0)
+
+
+def test_normalised_score_exact_sums_bit_exact():
+    """Confidence whose sums are exact in fp32 in any order (half-integers in pairs v, 15 - v): the long
+    reductions cannot depend on the summation order, so in bf16 the whole chain of rounded tensor operations
+    must reproduce the oracle's mask and window means bit for bit."""
+    g = torch.Generator().manual_seed(11)
+    batch, frames, H, W = 2, 4, 12, 12
+    half = torch.randint(0, 31, (batch, frames * H * W // 2), generator=g).float() / 2
+    conf = torch.cat([half, 15.0 - half], dim=1)[:, torch.randperm(frames * H * W, generator=g)]
+    conf = conf.reshape(batch * frames, H, W).bfloat16()
+    for thr in (-0.3, 0.0, 0.25):
+        mask, means = co_me_cuext.co_me_select_windows(conf.to(DEV), batch, 3, 3, thr, mode="mse", return_means=True)
+        want = oracle.select_lowest_confidence(conf, batch, 3, 3, thr, mode="mse")
+        flat = conf.reshape(batch, -1)
+        z = (flat - flat.mean(dim=-1, keepdim=True)) / (flat.std(dim=-1, keepdim=True) + 1e-3)
+        want_means = oracle.window_confidence_means(z.reshape(-1, H, W), 3, 3).float()
+        assert torch.equal(means.cpu(), want_means)
+        assert torch.equal(mask.cpu(), want)
+        assert 0 < int(want.sum()) < want.numel()
 
 
 def test_large_window_count_uses_the_global_path():
