@@ -42,7 +42,12 @@ def test_build_ctx_modes(B, S, H, W, G, mode, threshold):
     assert torch.equal(mask.cpu(), want)
     assert 0 < int(want.sum()) < want.numel()
     if mode == "pairwise-rank":
-        assert len(set(want.sum(dim=1).tolist())) == 1         # the same count in every frame: per-frame quantile
+        # per-frame quantile: frame 0, whose confidence is offset by +1, still merges its share; a joint quantile
+        # over the batch element (the 2-D merger's scope) would merge nothing there
+        joint = oracle.select_lowest_confidence(conf.reshape(B * S, 1, H * W), B, 1, G, threshold)
+        assert int(joint[0].sum()) == 0 and not torch.equal(joint, want)
+        if threshold == 0.5:
+            assert int(want[0].sum()) > 0
 
 
 def test_normalised_score_is_per_batch_element_not_per_frame():
