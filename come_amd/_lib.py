@@ -44,6 +44,10 @@ SIGNATURES = {
     "come_attn_varlen_fwd_ws": (_int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64,
                                        _ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _f32,
                                        _ptr, _i64, _i64, _ptr, _ptr, _i64, _ptr]),
+    "come_attn_static_work_bytes": (_i64, []),
+    "come_attn_varlen_fwd_static": (_int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64,
+                                           _ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _f32,
+                                           _ptr, _i64, _i64, _ptr, _ptr]),
     "come_qk_norm_rope": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                  _int, _ptr, _ptr, _ptr, _ptr, _f32, _ptr, _ptr, _ptr, _i64, _ptr]),
     "come_jagged_add_suffix": (_int, [_ptr, _ptr, _int, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr]),

@@ -25,6 +25,13 @@
 //   the segment get scores of -inf and probabilities of exactly 0.
 #include "come_common.h"
 
+#include <mutex>
+
+// Work buffer of come_attn_varlen_fwd_static: pieces of the key-split tail (unnormalised outputs, reference
+// points and row sums).  Every GPU the library runs on holds its own copy of the array at its own address.
+constexpr int64_t kStaticWorkBytes = 64ll << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticWorkBytes];
+
 namespace come {
 namespace {
 
@@ -818,13 +825,40 @@ extern "C" int64_t come_attn_work_bytes(int64_t n_seq, int64_t total, int64_t n_
     return make_plan(n_seq, total, n_heads, max_seqlen, true).work_bytes;
 }
 
-extern "C" int come_attn_varlen_fwd_ws(const void *q, const void *k, const void *v, int dtype, int64_t q_row_stride,
-                                       int64_t q_head_stride, int64_t k_row_stride, int64_t k_head_stride,
-                                       int64_t v_row_stride, int64_t v_head_stride, const int32_t *cu_seqlens,
-                                       int64_t n_seq, int64_t total, int64_t n_heads, int64_t head_dim,
-                                       const void *perkey_bias, int64_t max_seqlen, float softmax_scale, void *out,
-                                       int64_t o_row_stride, int64_t o_head_stride, float *lse, void *work,
-                                       int64_t work_bytes, void *stream) {
+// Address of this device's copy of `scratch` (nullptr + error message on failure).  The array's name is only a
+// host-side handle: the device address is asked for once per device, with that device current, and kept.
+static void *static_work_pointer() {
+    constexpr int kMaxDevices = 64;
+    static std::mutex lock;
+    static void *known[kMaxDevices] = {};
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error("come_attn_varlen_fwd_static: no usable current device (%s)", hipGetErrorString(e));
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> guard(lock);
+    if (known[dev] == nullptr) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr) {
+            set_error("come_attn_varlen_fwd_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        known[dev] = p;
+    }
+    return known[dev];
+}
+
+// Shared body of the three entry points.  static_work: the buffer is the library's own fixed-size array; a launch
+// that needs more is an error instead of a launch without the key split.
+static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int dtype, int64_t q_row_stride,
+                                int64_t q_head_stride, int64_t k_row_stride, int64_t k_head_stride,
+                                int64_t v_row_stride, int64_t v_head_stride, const int32_t *cu_seqlens,
+                                int64_t n_seq, int64_t total, int64_t n_heads, int64_t head_dim,
+                                const void *perkey_bias, int64_t max_seqlen, float softmax_scale, void *out,
+                                int64_t o_row_stride, int64_t o_head_stride, float *lse, void *work,
+                                int64_t work_bytes, bool static_work, void *stream) {
     clear_error();
     COME_REQUIRE(dtype == COME_BF16 || dtype == COME_F16, COME_ERR_UNSUPPORTED,
                  "come_attn_varlen_fwd: only fp16 and bf16 are supported");
@@ -856,7 +890,16 @@ extern "C" int come_attn_varlen_fwd_ws(const void *q, const void *k, const void 
                      (reinterpret_cast<uintptr_t>(v) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0,
                  COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: q/k/v must be 16-byte aligned, out 8-byte aligned");
 
-    Plan plan = make_plan(n_seq, total, n_heads, max_seqlen, work != nullptr);
+    Plan plan = make_plan(n_seq, total, n_heads, max_seqlen, work != nullptr || static_work);
+    if (static_work && plan.splits > 1) {
+        COME_REQUIRE(plan.work_bytes <= kStaticWorkBytes, COME_ERR_UNSUPPORTED,
+                     "come_attn_varlen_fwd_static: this launch needs a work buffer of %lld bytes, the built-in one "
+                     "holds %lld; use come_attn_varlen_fwd_ws with a buffer of come_attn_work_bytes() bytes",
+                     (long long)plan.work_bytes, (long long)kStaticWorkBytes);
+        work = static_work_pointer();
+        if (work == nullptr) return COME_ERR_HIP;
+        work_bytes = kStaticWorkBytes;
+    }
     if (plan.splits > 1 && (work_bytes < plan.work_bytes || (reinterpret_cast<uintptr_t>(work) & 15) != 0))
         plan = make_plan(n_seq, total, n_heads, max_seqlen, false);        // buffer too small or misaligned: no split
     const bool wide = plan.wide;
@@ -906,14 +949,42 @@ extern "C" int come_attn_varlen_fwd_ws(const void *q, const void *k, const void 
     return COME_OK;
 }
 
+extern "C" int come_attn_varlen_fwd_ws(const void *q, const void *k, const void *v, int dtype, int64_t q_row_stride,
+                                       int64_t q_head_stride, int64_t k_row_stride, int64_t k_head_stride,
+                                       int64_t v_row_stride, int64_t v_head_stride, const int32_t *cu_seqlens,
+                                       int64_t n_seq, int64_t total, int64_t n_heads, int64_t head_dim,
+                                       const void *perkey_bias, int64_t max_seqlen, float softmax_scale, void *out,
+                                       int64_t o_row_stride, int64_t o_head_stride, float *lse, void *work,
+                                       int64_t work_bytes, void *stream) {
+    return attn_varlen_fwd_impl(q, k, v, dtype, q_row_stride, q_head_stride, k_row_stride, k_head_stride,
+                                v_row_stride, v_head_stride, cu_seqlens, n_seq, total, n_heads, head_dim,
+                                perkey_bias, max_seqlen, softmax_scale, out, o_row_stride, o_head_stride, lse,
+                                work, work_bytes, false, stream);
+}
+
 extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v, int dtype, int64_t q_row_stride,
                                     int64_t q_head_stride, int64_t k_row_stride, int64_t k_head_stride,
                                     int64_t v_row_stride, int64_t v_head_stride, const int32_t *cu_seqlens,
                                     int64_t n_seq, int64_t total, int64_t n_heads, int64_t head_dim,
                                     const void *perkey_bias, int64_t max_seqlen, float softmax_scale, void *out,
                                     int64_t o_row_stride, int64_t o_head_stride, float *lse, void *stream) {
-    return come_attn_varlen_fwd_ws(q, k, v, dtype, q_row_stride, q_head_stride, k_row_stride, k_head_stride,
-                                   v_row_stride, v_head_stride, cu_seqlens, n_seq, total, n_heads, head_dim,
-                                   perkey_bias, max_seqlen, softmax_scale, out, o_row_stride, o_head_stride, lse,
-                                   nullptr, 0, stream);
+    return attn_varlen_fwd_impl(q, k, v, dtype, q_row_stride, q_head_stride, k_row_stride, k_head_stride,
+                                v_row_stride, v_head_stride, cu_seqlens, n_seq, total, n_heads, head_dim,
+                                perkey_bias, max_seqlen, softmax_scale, out, o_row_stride, o_head_stride, lse,
+                                nullptr, 0, false, stream);
+}
+
+extern "C" int64_t come_attn_static_work_bytes(void) { return kStaticWorkBytes; }
+
+extern "C" int come_attn_varlen_fwd_static(const void *q, const void *k, const void *v, int dtype,
+                                           int64_t q_row_stride, int64_t q_head_stride, int64_t k_row_stride,
+                                           int64_t k_head_stride, int64_t v_row_stride, int64_t v_head_stride,
+                                           const int32_t *cu_seqlens, int64_t n_seq, int64_t total, int64_t n_heads,
+                                           int64_t head_dim, const void *perkey_bias, int64_t max_seqlen,
+                                           float softmax_scale, void *out, int64_t o_row_stride,
+                                           int64_t o_head_stride, float *lse, void *stream) {
+    return attn_varlen_fwd_impl(q, k, v, dtype, q_row_stride, q_head_stride, k_row_stride, k_head_stride,
+                                v_row_stride, v_head_stride, cu_seqlens, n_seq, total, n_heads, head_dim,
+                                perkey_bias, max_seqlen, softmax_scale, out, o_row_stride, o_head_stride, lse,
+                                nullptr, 0, true, stream);
 }

@@ -220,6 +220,32 @@ int come_attn_varlen_fwd_ws(const void *q, const void *k, const void *v, int dty
                             float *lse, void *work, int64_t work_bytes, void *stream);
 
 /*
+ * come_attn_varlen_fwd_static — come_attn_varlen_fwd_ws without a buffer argument and without any allocation:
+ * the pieces of the key-split tail go to a fixed array of come_attn_static_work_bytes() bytes (64 MiB) that is part
+ * of the library's device image, one copy per GPU, held until the process ends.  Same kernels, same launch shape
+ * and therefore the same results as come_attn_varlen_fwd_ws with a buffer of come_attn_work_bytes(...) bytes.
+ *
+ * A launch whose come_attn_work_bytes(...) exceeds come_attn_static_work_bytes() fails with COME_ERR_UNSUPPORTED
+ * (nothing is enqueued).  All calls on one GPU share that GPU's array: calls that may run concurrently there (on
+ * different streams or from different threads) race on it and must be serialised by the caller; calls on one
+ * stream are ordered by the stream.  Nothing in the array has to be cleared between calls: every piece is
+ * written in full before the combining kernel of the same call reads it.
+ *
+ * No counterpart in the reference.  It is for callers that cannot allocate device memory around the call: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid allocation.
+ */
+int64_t come_attn_static_work_bytes(void);
+int come_attn_varlen_fwd_static(const void *q, const void *k, const void *v, int dtype,
+                                int64_t q_row_stride, int64_t q_head_stride,
+                                int64_t k_row_stride, int64_t k_head_stride,
+                                int64_t v_row_stride, int64_t v_head_stride,
+                                const int32_t *cu_seqlens, int64_t n_seq, int64_t total,
+                                int64_t n_heads, int64_t head_dim,
+                                const void *perkey_bias, int64_t max_seqlen, float softmax_scale,
+                                void *out, int64_t o_row_stride, int64_t o_head_stride,
+                                float *lse, void *stream);
+
+/*
  * come_qk_norm_rope — attention prologue, in place on the packed projection output:
  * LayerNorm over the head dimension of every q and k head, then the 2-D rotary position
  * embedding.
