@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "power", "prologue", "shapes", "copy", "e2e", "stress", "stress_e2e", "frame"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "prologue", "copy", "e2e", "stress", "stress_e2e", "frame"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -426,85 +426,6 @@ def bench_bias_overhead(device):
     return out
 
 
-def bench_power(device, seconds=4.0):
-    """Board power (hwmon ``power1_input`` / ``power1_average`` of the GPU, sampled every 20 ms from sysfs) while
-    the headline attention launch and the library bf16 GEMM run back to back for ``seconds`` each, on N(0,1) and on
-    all-zero operands.  Shows which of the two limits a kernel runs into: its own schedule or the power cap."""
-    import glob
-    import threading
-
-    import torch
-    from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
-
-    files = {}
-    for name in ("power1_average", "power1_input", "power1_cap"):
-        files[name] = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/" + name))
-
-    def read(name):
-        vals = []
-        for f in files.get(name, []):
-            try:
-                with open(f) as fh:
-                    vals.append(int(fh.read().strip()))
-            except (OSError, ValueError):
-                pass
-        return vals
-
-    def watts():
-        vals = read("power1_average") or read("power1_input")
-        return max(vals) / 1e6 if vals else None
-
-    def phase(fn, flops):
-        samples, stop = [], threading.Event()
-
-        def sampler():
-            while not stop.is_set():
-                samples.append(watts())
-                time.sleep(0.02)
-
-        t = threading.Thread(target=sampler)
-        t.start()
-        t0, calls = time.perf_counter(), 0
-        while time.perf_counter() - t0 < seconds:
-            if fn is None:
-                time.sleep(0.05)
-            else:
-                for _ in range(10):
-                    fn()
-                torch.cuda.synchronize()
-                calls += 10
-        dt = time.perf_counter() - t0
-        stop.set()
-        t.join()
-        steady = [x for x in samples[len(samples) // 3:] if x is not None]
-        out = {"power_W": round(sum(steady) / len(steady), 1) if steady else None}
-        if calls:
-            out.update(ms_per_call=round(dt / calls * 1e3, 3), TFLOPs=round(flops * calls / dt / 1e12, 1))
-        return out
-
-    w = make_attention_workload(device)
-    zeros = torch.zeros_like(w["qkv"])
-    max_len = max(w["lens"])
-    a = torch.randn(8192, 8192, device=device).bfloat16()
-    b = torch.randn(8192, 8192, device=device).bfloat16()
-    z = torch.zeros_like(a)
-    cap = read("power1_cap")
-
-    def attn(qkv):
-        return lambda: flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, w["cu"], max_len, perkey_bias=w["bias"],
-                                                                      softmax_scale=0.125)
-
-    only_v, only_qk = zeros.clone(), w["qkv"].clone()
-    only_v[:, 2] = w["qkv"][:, 2]
-    only_qk[:, 2] = 0
-
-    return {"power_cap_W": max(cap) / 1e6 if cap else None, "idle": phase(None, 0),
-            "attention_normal": phase(attn(w["qkv"]), w["flops"]), "attention_zeros": phase(attn(zeros), w["flops"]),
-            "attention_only_v_normal": phase(attn(only_v), w["flops"]),
-            "attention_only_qk_normal": phase(attn(only_qk), w["flops"]),
-            "gemm_8192_normal": phase(lambda: a @ b, 2.0 * 8192 ** 3), "gemm_8192_zeros": phase(lambda: z @ z, 2.0 * 8192 ** 3)}
-
-
 def bench_qk_prologue(device, rows=(25536, 43968), iters=200, warmup=20):
     """q / k LayerNorm + 2-D RoPE in place on the packed ``qkv [P, 3, 16, 64]`` bf16 (one launch through the C ABI),
     over 4 rotating tensors (each launch touches 2/3 of 157 MB at P = 25 536).  Algorithmic bytes: q and k read and
@@ -539,40 +460,6 @@ def bench_qk_prologue(device, rows=(25536, 43968), iters=200, warmup=20):
                            "frac": round(gbs / PEAK_HBM_GBS, 4)}
         del sets
         torch.cuda.empty_cache()
-    return out
-
-
-def bench_attention_shapes(device):
-    """The attention kernel on other shapes than the headline one (16 heads x 64, bf16, counts of 1): single long
-    segments (key-split tail), several equal segments, short segments as in frame attention, and the headline
-    workload with q and k scaled up (sharper logits make the rare reference-point path more frequent)."""
-    import torch
-    from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
-
-    g = torch.Generator().manual_seed(0)
-    frames = torch.randint(686, 863, (32,), generator=g).tolist()
-    stress = torch.randint(305, 482, (128,), generator=g).tolist()
-    cases = {"1 x 25536": [25536], "1 x 21848": [21848], "1 x 43968": [43968], "1 x 49960": [49960],
-             "4 x 12768": [12768] * 4, "2 x 25536": [25536] * 2, "8 x 3000": [3000] * 8, "16 x 2048": [2048] * 16,
-             "32 x 1374": [1374] * 32, "128 x 1041": [1041] * 128, "32 x 800": [800] * 32, "32 x 768": [768] * 32,
-             "32 x U[686,862]": frames, "128 x U[305,481]": stress}
-    out = {}
-    for name, lens in cases.items():
-        steps = 20 if sum(lens) > 20000 and max(lens) > 4000 else 50
-        ms, tflops, _ = attention_case(device, lens, torch.ones(sum(lens)), steps=steps, warmup=5)
-        out[name] = {"us_per_call": round(ms * 1e3, 1), "TFLOPs": round(tflops, 1)}
-    w = make_attention_workload(device)
-    base, max_len = w["qkv"].float(), max(w["lens"])
-    sharp = {}
-    for scale in (1.0, 2.0, 2.83, 4.0):
-        x = base.clone()
-        x[:, :2] *= scale
-        x = x.bfloat16()
-        _, ms = time_loop(lambda: flash_attn_varlen_qkvpacked_func_w_perkey_bias(x, w["cu"], max_len, perkey_bias=w["bias"],
-                                                                                 softmax_scale=0.125), 10, 3)
-        sharp["logit sigma %.0f nats" % (scale * scale)] = {"ms_per_call": round(ms / 10, 3),
-                                                            "TFLOPs": round(w["flops"] / (ms / 10 * 1e-3) / 1e12, 1)}
-    out["headline workload, q and k scaled"] = sharp
     return out
 
 
@@ -779,10 +666,6 @@ def main():
             w, wall, ev_ms = bench_attention(args.steps, args.warmup, device)
             print(json.dumps({"only": "attn", "ms_per_call": ev_ms / args.steps,
                               "tflops": w["flops"] / (ev_ms / args.steps * 1e-3) / 1e12}))
-        elif args.only == "power":                               # 20 s of sustained load: not part of the default run
-            print(json.dumps({"only": "power", **bench_power(device)}))
-        elif args.only == "shapes":                              # about 20 s: not part of the default run
-            print(json.dumps({"only": "shapes", **bench_attention_shapes(device)}))
         elif args.only == "prologue":
             print(json.dumps({"only": "prologue", **bench_qk_prologue(device, iters=args.steps, warmup=args.warmup)}))
         elif args.only == "refmerge":

@@ -381,6 +381,66 @@ __global__ __launch_bounds__(kThreads) void split_vec_kernel(const uint4 *__rest
         if (i0 + r < total) st16_stream(out + (i0 + r) * out_chunks + out_chunk, v[r]);
 }
 
+// Wave-per-row form for rows that are a multiple of 1 KiB wide (64 chunks): a wavefront owns ROWS consecutive
+// output rows x one 64-chunk (1 KiB) column segment.  The row index is wave-uniform, so the indices come through the
+// scalar path (one s_load for all of the wavefront's rows, no vector load in front of the gather) and the
+// wavefront's row loads are issued back to back before the first store.  Measured on 16 / 32 / 64 / 128 frames:
+// one row per wavefront is best while the launch is a few rounds of wavefronts (more, shorter wavefronts drain
+// evenly), two rows from about 64 k wavefronts on (+9 .. 15 %); four and eight rows are slower everywhere.
+constexpr int kSplitWaves = 4;
+
+template <typename IndexT, bool PAIR, int ROWS>
+__global__ __launch_bounds__(64 * kSplitWaves) void split_wave_kernel(const uint4 *__restrict__ merged,
+                                                                      const uint4 *__restrict__ merged_b,
+                                                                      int64_t merged_rows,
+                                                                      const IndexT *__restrict__ rev, int total,
+                                                                      int chunks, uint4 *__restrict__ out,
+                                                                      int segs, uint32_t n_waves, uint32_t run,
+                                                                      uint32_t remapped_blocks, FastDiv by_run,
+                                                                      FastDiv by_segs) {
+    uint32_t bid = blockIdx.x;
+    if (bid < remapped_blocks) {                            // runs of `run` workgroups stay on one XCD (one L2)
+        const uint32_t local = bid >> 3;
+        const uint32_t q = fast_div(local, by_run);
+        bid = (q * 8u + (bid & 7u)) * run + (local - q * run);
+    }
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(bid * kSplitWaves + (threadIdx.x >> 6));
+    if (wave >= n_waves) return;
+    const int lane = threadIdx.x & 63;
+    const uint32_t group = fast_div(wave, by_segs);
+    const int seg = static_cast<int>(wave - group * segs);
+    const int row0 = static_cast<int>(group) * ROWS;
+    const int out_chunks = PAIR ? 2 * chunks : chunks;
+    const int out_chunk = seg * 64 + lane;
+    const bool second = PAIR && seg * 64 >= chunks;          // wave-uniform: chunks is a multiple of 64
+    const uint4 *__restrict__ src = second ? merged_b : merged;
+    const int chunk = second ? out_chunk - chunks : out_chunk;
+    uint4 *__restrict__ dst = out + static_cast<int64_t>(row0) * out_chunks + out_chunk;
+    if (row0 + ROWS <= total) {
+        // all indices first, then all row loads, then the stores: the wavefront's ROWS index -> row -> store
+        // chains overlap instead of running one after the other
+        int64_t s[ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) s[r] = static_cast<int64_t>(rev[row0 + r]);
+        uint4 v[ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            const bool ok = s[r] >= 0 && s[r] < merged_rows;
+            v[r] = src[(ok ? s[r] : 0) * chunks + chunk];
+            if (!ok) v[r] = make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) st16_stream(dst + static_cast<int64_t>(r) * out_chunks, v[r]);
+        return;
+    }
+    for (int r = 0; row0 + r < total; ++r) {                 // the last, partial group of rows
+        const int64_t s = static_cast<int64_t>(rev[row0 + r]);
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (s >= 0 && s < merged_rows) v = src[s * chunks + chunk];
+        st16_stream(dst + static_cast<int64_t>(r) * out_chunks, v);
+    }
+}
+
 // element-wise fallback; `pair`: output rows are [row of merged | row of merged_b]
 template <typename IndexT>
 __global__ __launch_bounds__(kThreads) void split_elem_kernel(const uint8_t *__restrict__ merged,
@@ -588,6 +648,33 @@ static int token_split_impl(const char *who, bool pair, const void *merged, cons
         for (int64_t r0 = 0; r0 < total; r0 += rows_per_launch) {
             const int64_t nr = total - r0 < rows_per_launch ? total - r0 : rows_per_launch;
             const int64_t items = nr * out_chunks;
+            if (out_chunks % 64 == 0 && chunks % 64 == 0 && merged_rows > 0) {
+                const int segs = out_chunks / 64;
+                const int wave_rows = nr * segs > 65536 ? 2 : 1;
+                const int64_t n_waves = ceil_div(nr, wave_rows) * segs;
+                const int64_t wrun64 = static_cast<int64_t>(kSplitRunRows) / wave_rows * segs / kSplitWaves;
+                const uint32_t wrun = static_cast<uint32_t>(wrun64 < 1 ? 1 : wrun64);
+                const dim3 wgrid(static_cast<unsigned>(ceil_div(n_waves, kSplitWaves))), wblock(64 * kSplitWaves);
+                const uint4 *a4 = static_cast<const uint4 *>(merged), *b4 = static_cast<const uint4 *>(merged_b);
+                uint4 *o4 = static_cast<uint4 *>(out) + r0 * out_chunks;
+#define COME_SPLITW_ROWS(IDX_, PAIR_, REV_, ROWS_)                                                                  \
+    hipLaunchKernelGGL((split_wave_kernel<IDX_, PAIR_, ROWS_>), wgrid, wblock, 0, s, a4, b4, merged_rows,           \
+                       REV_ + r0, static_cast<int>(nr), chunks, o4, segs, static_cast<uint32_t>(n_waves), wrun,     \
+                       (wgrid.x / (8u * wrun)) * (8u * wrun), make_fastdiv(wrun), make_fastdiv(segs))
+#define COME_SPLITW_CASE(IDX_, PAIR_, REV_)                                 \
+    do {                                                                    \
+        if (wave_rows == 2) COME_SPLITW_ROWS(IDX_, PAIR_, REV_, 2);         \
+        else COME_SPLITW_ROWS(IDX_, PAIR_, REV_, 1);                        \
+    } while (0)
+                if (rev_i64 && pair) COME_SPLITW_CASE(int64_t, true, rev_i64);
+                else if (rev_i64) COME_SPLITW_CASE(int64_t, false, rev_i64);
+                else if (pair) COME_SPLITW_CASE(int32_t, true, rev_i32);
+                else COME_SPLITW_CASE(int32_t, false, rev_i32);
+#undef COME_SPLITW_CASE
+#undef COME_SPLITW_ROWS
+                COME_CHECK_LAUNCH(who);
+                continue;
+            }
             const dim3 grid(static_cast<unsigned>(ceil_div(items, kThreads))), block(kThreads);
             const uint4 *a4 = static_cast<const uint4 *>(merged), *b4 = static_cast<const uint4 *>(merged_b);
             uint4 *o4 = static_cast<uint4 *>(out) + r0 * out_chunks;

@@ -211,6 +211,32 @@ def test_split_pair_edges_and_errors():
         co_me_cuext.co_me_token_split_pair_cuda(a, b, rev.float(), C)
 
 
+@pytest.mark.parametrize("index_dtype", [torch.int64, torch.int32], ids=["i64", "i32"])
+@pytest.mark.parametrize("dtype,C,total", [(torch.bfloat16, 512, 1001), (torch.bfloat16, 1024, 777), (torch.float32, 256, 333),
+                                           (torch.bfloat16, 512, 70001), (torch.float32, 1024, 16401),
+                                           (torch.float16, 1536, 21851)],
+                         ids=["bf16-1seg", "bf16-2seg", "fp32-1seg", "bf16-two-rows-odd", "fp32-two-rows-odd", "fp16-3seg"])
+def test_split_rows_of_whole_kibibytes(dtype, C, total, index_dtype):
+    """Rows that are a multiple of 1 KiB wide take the wavefront-per-row kernel (one or two rows per wavefront
+    depending on the launch size; an odd row count leaves a partial last group).  Indices outside the packed
+    rows give rows of zeros."""
+    P = 999
+    g = torch.Generator().manual_seed(total)
+    a = torch.randn(P, C, generator=g).to(dtype)
+    b = torch.randn(P, C, generator=g).to(dtype)
+    rev = torch.randint(0, P, (total,), generator=g)
+    rev[[0, 5, total // 2, total - 1]] = torch.tensor([P - 1, -1, P, 0])
+    rev[7] = 2 ** 40 if index_dtype == torch.int64 else 2 ** 31 - 1
+    valid = (rev >= 0) & (rev < P)
+    want_a = torch.where(valid[:, None], a[rev.clamp(0, P - 1)], torch.zeros((), dtype=dtype))
+    want_b = torch.where(valid[:, None], b[rev.clamp(0, P - 1)], torch.zeros((), dtype=dtype))
+    a_d, b_d, rev_d = a.to(DEV), b.to(DEV), rev.to(index_dtype).to(DEV)
+    got = co_me_cuext.co_me_token_split_cuda(a_d, rev_d, C)
+    assert torch.equal(got.cpu(), want_a)
+    pair = co_me_cuext.co_me_token_split_pair_cuda(a_d, b_d, rev_d, C)
+    assert torch.equal(pair.cpu(), torch.cat((want_a, want_b), dim=-1))
+
+
 def test_split_pair_full_size_through_the_merger():
     from come_amd.token_merger import func_token_split_pair
     B, H, W, S, C = 16, 37, 37, 5, 1024
