@@ -192,11 +192,13 @@ def merge_workload(device, ratio=0.5, sets=None, frames=16, H=37, W=37, jitter=N
         mask.copy_(jittered_frame_masks(conf.cpu(), ratio, jitter, seed=1).to(torch.uint8))
 
     def select_and_plan():
-        if jitter is None:
-            _lib.check(lib.come_select_windows(conf.data_ptr(), _lib.COME_F32, 1, frames, H, W, 3, 3, 0, ratio,
-                                               means.data_ptr(), mask.data_ptr(), None, 0, stream))
-        _lib.check(lib.come_merge_plan(mask.data_ptr(), frames, M, S0, 9, tail, offsets.data_ptr(),
-                                       prefix.data_ptr(), stream))
+        if jitter is None:         # confidence -> mask -> plan in one launch
+            _lib.check(lib.come_select_plan(conf.data_ptr(), _lib.COME_F32, 1, frames, H, W, 3, 3, 0, ratio, S0,
+                                            means.data_ptr(), mask.data_ptr(), offsets.data_ptr(), prefix.data_ptr(),
+                                            None, 0, stream))
+        else:
+            _lib.check(lib.come_merge_plan(mask.data_ptr(), frames, M, S0, 9, tail, offsets.data_ptr(),
+                                           prefix.data_ptr(), stream))
 
     select_and_plan()
     P = int(offsets[-1].item())

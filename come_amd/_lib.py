@@ -36,6 +36,8 @@ SIGNATURES = {
     "come_token_split_pair": (_int, [_ptr, _ptr, _int, _i64, _i64, _ptr, _ptr, _i64, _ptr, _ptr]),
     "come_select_windows": (_int, [_ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int, _f32,
                                    _ptr, _ptr, _ptr, _i64, _ptr]),
+    "come_select_plan": (_int, [_ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int, _f32, _i64,
+                                _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr]),
     "come_select_work_bytes": (_i64, [_i64, _i64, _i64, _i64, _i64, _i64]),
     "come_attn_varlen_fwd": (_int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64,
                                     _ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _f32,

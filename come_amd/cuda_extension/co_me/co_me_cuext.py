@@ -32,17 +32,21 @@ def _torch_check(cond: bool, msg: str) -> None:
         raise RuntimeError(msg)
 
 
-def _merge_impl(tokens, start_index, gh, gw, H, W, mask_u8, n_groups, tail, index_dtype, count_dtype):
-    """plan -> read P -> allocate -> merge.  Returns (out, offsets_i32, index_map, counts)."""
+def _merge_impl(tokens, start_index, gh, gw, H, W, mask_u8, n_groups, tail, index_dtype, count_dtype, planned=None):
+    """plan -> read P -> allocate -> merge.  Returns (out, offsets_i32, index_map, counts).
+    ``planned = (offsets, prefix)``: the plan was already made on the device (``come_select_plan``)."""
     lib = _lib.load()
     dev = tokens.device
     B, N, C = tokens.shape
     with torch.cuda.device(dev):
         stream = _lib.current_stream(dev)
-        offsets = torch.empty(B + 1, dtype=torch.int32, device=dev)
-        prefix = torch.empty(B, max(n_groups, 1), dtype=torch.int32, device=dev)
-        _lib.check(lib.come_merge_plan(_lib.ptr(mask_u8), B, n_groups, start_index, gh * gw, tail,
-                                       offsets.data_ptr(), prefix.data_ptr(), stream))
+        if planned is None:
+            offsets = torch.empty(B + 1, dtype=torch.int32, device=dev)
+            prefix = torch.empty(B, max(n_groups, 1), dtype=torch.int32, device=dev)
+            _lib.check(lib.come_merge_plan(_lib.ptr(mask_u8), B, n_groups, start_index, gh * gw, tail,
+                                           offsets.data_ptr(), prefix.data_ptr(), stream))
+        else:
+            offsets, prefix = planned
         P = int(offsets[-1].item()) if B > 0 else 0          # the one host sync (output shape)
         out = torch.empty(P, C, dtype=tokens.dtype, device=dev)
         index_map = torch.empty(B * N, dtype=index_dtype, device=dev)
@@ -193,12 +197,41 @@ def co_me_select_windows(conf: torch.Tensor, batch: int, group_h: int, group_w: 
 
 def co_me_select_merge_2d(tokens: torch.Tensor, conf: torch.Tensor, batch: int, start_index: int, group_h: int,
                           group_w: int, H: int, W: int, ratio: float, index_dtype: torch.dtype = torch.int32,
-                          count_dtype: torch.dtype = torch.int32):
+                          count_dtype: torch.dtype = torch.int32, mode: str = "pairwise-rank"):
     """Confidence-guided merge in one call: window means -> joint lowest-``ratio`` selection per
-    batch element -> gather-mean.  Returns
+    batch element -> merge plan (one launch for all three when ``batch == 1``) -> gather-mean.  Returns
     ``(merged [P,C], index_map [B_eff*N], counts [P], cu_seqlens [B_eff+1] int32, mask [B_eff,M] bool)``.
     """
-    mask = co_me_select_windows(conf.reshape(-1, H, W), batch, group_h, group_w, ratio)
-    out, offsets, index_map, counts = co_me_token_merge_2d_cuda(tokens, start_index, group_h, group_w, H, W, mask,
-                                                                 index_dtype=index_dtype, count_dtype=count_dtype)
+    _torch_check(tokens.is_cuda and conf.is_cuda, "tokens and conf must be on CUDA")
+    _torch_check(tokens.dim() == 3, "tokens must be [B, N, C]")
+    _torch_check(mode in _MODES, f"unsupported confidence mode {mode!r}")
+    _torch_check(conf.dtype in (torch.bfloat16, torch.float32), "conf must be bfloat16 or float32")
+    start_index, group_h, group_w, H, W = int(start_index), int(group_h), int(group_w), int(H), int(W)
+    _torch_check(start_index >= 0 and group_h > 0 and group_w > 0 and H >= 0 and W >= 0, "bad geometry")
+    rows, N, _ = tokens.shape
+    M = (H // group_h) * (W // group_w)
+    _torch_check(N == start_index + H * W, "N != start_index + H * W")
+    _torch_check(batch > 0 and rows % batch == 0, "token rows must be a multiple of batch")
+    _torch_check(conf.numel() == rows * H * W, "conf must hold one value per grid position")
+    if M == 0 or rows == 0:         # nothing to select from: every token is kept
+        mask = torch.zeros(rows, M, dtype=torch.bool, device=tokens.device)
+        out, offsets, index_map, counts = co_me_token_merge_2d_cuda(tokens, start_index, group_h, group_w, H, W, mask,
+                                                                     index_dtype=index_dtype, count_dtype=count_dtype)
+        return out, index_map, counts, offsets, mask
+    lib = _lib.load()
+    dev = tokens.device
+    tokens_c = tokens.contiguous()
+    conf_c = conf.reshape(rows, H, W).contiguous()
+    with torch.cuda.device(dev):
+        mask = torch.empty(rows, M, dtype=torch.bool, device=dev)
+        means = torch.empty(rows, M, dtype=torch.float32, device=dev)
+        offsets = torch.empty(rows + 1, dtype=torch.int32, device=dev)
+        prefix = torch.empty(rows, M, dtype=torch.int32, device=dev)
+        _lib.check(lib.come_select_plan(conf_c.data_ptr(), _lib.dtype_code(conf_c.dtype), batch, rows // batch, H, W,
+                                        group_h, group_w, _MODES[mode], float(ratio), start_index, means.data_ptr(),
+                                        mask.data_ptr(), offsets.data_ptr(), prefix.data_ptr(), None, 0,
+                                        _lib.current_stream(dev)))
+    tail = H * W - M * group_h * group_w
+    out, offsets, index_map, counts = _merge_impl(tokens_c, start_index, group_h, group_w, H, W, mask.view(torch.uint8),
+                                                  M, tail, index_dtype, count_dtype, planned=(offsets, prefix))
     return out, index_map, counts, offsets, mask

@@ -162,6 +162,27 @@ int64_t come_select_work_bytes(int64_t batch, int64_t frames, int64_t grid_h, in
                                int64_t group_h, int64_t group_w);
 
 /*
+ * come_select_plan — come_select_windows followed by come_merge_plan of the selected mask, in one launch when
+ * batch == 1 (the mask never leaves the workgroup that made it; with batch > 1 a second, one-wavefront launch scans
+ * the row lengths into offsets).
+ *
+ *   arguments up to merge_mask as for come_select_windows; start_index as for come_merge_plan
+ *   offsets      [batch * frames + 1] int32 out, group_prefix [batch * frames, windows] int32 out: exactly what
+ *                come_merge_plan(merge_mask, batch * frames, windows, start_index, group_h * group_w,
+ *                grid_h * grid_w - windows * group_h * group_w, ...) writes
+ * The grid must hold at least one full window.
+ *
+ * Stands in for build_ctx's selection (src/accelerate/token_merger/co_me_2d.py:268-298) plus the scan + cumsum
+ * front end of the merge (src/cuda_extension/co_me/src/kernel_token_merge.cu:12-46, 271-286), which the reference
+ * runs as torch.quantile's sort, a dozen small tensor kernels and two host reads.
+ */
+int come_select_plan(const void *conf, int dtype, int64_t batch, int64_t frames,
+                     int64_t grid_h, int64_t grid_w, int64_t group_h, int64_t group_w,
+                     int mode, float threshold, int64_t start_index,
+                     float *means_f32, uint8_t *merge_mask, int32_t *offsets, int32_t *group_prefix,
+                     void *work, int64_t work_bytes, void *stream);
+
+/*
  * come_attn_varlen_fwd — softmax(Q K^T * softmax_scale + bias[key]) V per packed
  * segment and head, forward only, no causal mask, no dropout.
  *

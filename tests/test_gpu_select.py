@@ -155,13 +155,86 @@ def test_normalised_score_exact_sums_bit_exact():
 
 
 def test_large_window_count_uses_the_global_path():
-    # more than 8192 windows per batch element: the means no longer fit the per-thread registers
-    conf = torch.rand(40, 45, 45, generator=torch.Generator().manual_seed(7))     # 40 * 225 = 9000 windows
+    # more than 16384 windows per batch element: the means no longer fit the per-thread registers
+    conf = torch.rand(80, 45, 45, generator=torch.Generator().manual_seed(7))     # 80 * 225 = 18000 windows
     for ratio in (0.3, 0.62):
         mask = co_me_cuext.co_me_select_windows(conf.to(DEV), 1, 3, 3, ratio)
         gpu_means = co_me_cuext.co_me_select_windows(conf.to(DEV), 1, 3, 3, ratio, return_means=True)[1].cpu()
         cut = torch.quantile(gpu_means.reshape(1, -1), ratio, dim=-1, keepdim=True)
         assert torch.equal(mask.cpu().reshape(1, -1), gpu_means.reshape(1, -1) < cut)
+
+
+def _select_plan(conf, batch, gh, gw, threshold, start_index, mode=0):
+    """come_select_plan through the C ABI -> (mask, means, offsets, prefix)."""
+    from come_amd import _lib
+    lib = _lib.load()
+    rows, H, W = conf.shape
+    M = (H // gh) * (W // gw)
+    mask = torch.empty(rows, M, dtype=torch.bool, device=DEV)
+    means = torch.empty(rows, M, dtype=torch.float32, device=DEV)
+    offsets = torch.full((rows + 1,), -7, dtype=torch.int32, device=DEV)
+    prefix = torch.full((rows, M), -7, dtype=torch.int32, device=DEV)
+    _lib.check(lib.come_select_plan(conf.data_ptr(), _lib.dtype_code(conf.dtype), batch, rows // batch, H, W, gh, gw,
+                                    mode, threshold, start_index, means.data_ptr(), mask.data_ptr(), offsets.data_ptr(),
+                                    prefix.data_ptr(), None, 0, _lib.current_stream(conf.device)))
+    return mask, means, offsets, prefix
+
+
+def _plan(mask, start_index, G, tail):
+    from come_amd import _lib
+    lib = _lib.load()
+    rows, M = mask.shape
+    offsets = torch.empty(rows + 1, dtype=torch.int32, device=DEV)
+    prefix = torch.empty(rows, M, dtype=torch.int32, device=DEV)
+    _lib.check(lib.come_merge_plan(mask.view(torch.uint8).data_ptr(), rows, M, start_index, G, tail, offsets.data_ptr(),
+                                   prefix.data_ptr(), _lib.current_stream(mask.device)))
+    return offsets, prefix
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+@pytest.mark.parametrize("batch,frames,H,W,gh,gw,ratio", [(1, 16, 37, 37, 3, 3, 0.5), (1, 128, 37, 28, 3, 3, 0.75),
+                                                          (1, 1, 6, 6, 3, 3, 0.5), (3, 4, 12, 9, 3, 3, 0.37),
+                                                          (2, 20, 37, 37, 3, 3, 0.25), (1, 80, 45, 45, 3, 3, 0.62),
+                                                          (1, 7, 20, 16, 2, 4, 0.4), (2, 3, 1, 64, 1, 4, 0.5)])
+def test_select_plan_is_select_then_plan(batch, frames, H, W, gh, gw, ratio, dtype):
+    """One launch from the confidence to the merge plan: mask and means as come_select_windows gives them, offsets
+    and prefix as come_merge_plan gives them for that mask, and against the closed form of the offsets."""
+    conf = _smooth_confidence(batch * frames, H, W, seed=frames + W).to(dtype).to(DEV)
+    S0 = 5
+    mask, means, offsets, prefix = _select_plan(conf, batch, gh, gw, ratio, S0)
+    mask_ref, means_ref = co_me_cuext.co_me_select_windows(conf, batch, gh, gw, ratio, return_means=True)
+    assert torch.equal(mask, mask_ref) and torch.equal(means, means_ref)
+    if gh == 3 and gw == 3 and dtype == torch.bfloat16:
+        assert torch.equal(mask.cpu(), oracle.select_lowest_confidence(conf.cpu(), batch, 3, 3, ratio))
+    G = gh * gw
+    M = (H // gh) * (W // gw)
+    tail = H * W - M * G
+    offsets_ref, prefix_ref = _plan(mask, S0, G, tail)
+    assert torch.equal(offsets, offsets_ref)
+    assert torch.equal(prefix, prefix_ref)
+    lens = S0 + tail + M * G - (G - 1) * mask.sum(dim=1)
+    assert torch.equal(offsets.cpu().long(), torch.cat((torch.zeros(1, dtype=torch.long), lens.cpu().cumsum(0))))
+
+
+def test_select_plan_other_modes_and_errors():
+    from come_amd import _lib
+    conf = torch.rand(8, 12, 12, generator=torch.Generator().manual_seed(5)).to(DEV)
+    for mode, name, thr in ((1, "abs_mse", 0.5), (2, "mse", 0.0)):
+        mask, _, offsets, prefix = _select_plan(conf, 2, 3, 3, thr, 0, mode=mode)
+        assert torch.equal(mask, co_me_cuext.co_me_select_windows(conf, 2, 3, 3, thr, mode=name))
+        o_ref, p_ref = _plan(mask, 0, 9, 0)
+        assert torch.equal(offsets, o_ref) and torch.equal(prefix, p_ref)
+    lib = _lib.load()
+    small = torch.rand(2, 2, 2, device=DEV)                       # no full 3x3 window
+    dummy = torch.empty(16, dtype=torch.int32, device=DEV)
+    rc = lib.come_select_plan(small.data_ptr(), 0, 1, 2, 2, 2, 3, 3, 0, 0.5, 0, dummy.data_ptr(), dummy.data_ptr(),
+                              dummy.data_ptr(), dummy.data_ptr(), None, 0, None)
+    assert rc == 2 and b"no full window" in lib.come_last_error()
+    # the Python operator handles that case by keeping every token
+    tokens = torch.randn(2, 5 + 4, 64, device=DEV).bfloat16()
+    merged, index_map, counts, cu, mask = co_me_cuext.co_me_select_merge_2d(tokens, small, 1, 5, 3, 3, 2, 2, 0.5)
+    assert torch.equal(merged, tokens.reshape(-1, 64)) and cu.tolist() == [0, 9, 18] and mask.shape == (2, 0)
+    assert torch.equal(index_map.cpu(), torch.arange(18, dtype=torch.int32)) and bool((counts == 1).all())
 
 
 @pytest.mark.parametrize("ratio", [0.25, 0.5, 0.75])
