@@ -43,6 +43,7 @@ SIGNATURES = {
                                     _ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _f32,
                                     _ptr, _i64, _i64, _ptr, _ptr]),
     "come_attn_work_bytes": (_i64, [_i64, _i64, _i64, _i64]),
+    "come_attn_set_exact_scale": (_int, [_int]),
     "come_attn_varlen_fwd_ws": (_int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64,
                                        _ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _f32,
                                        _ptr, _i64, _i64, _ptr, _ptr, _i64, _ptr]),
@@ -78,6 +79,8 @@ def load() -> ctypes.CDLL:
                 fn = getattr(lib, name)
                 fn.restype = restype
                 fn.argtypes = argtypes
+            if os.environ.get("COME_ATTN_EXACT_SCALE", "0") not in ("", "0"):
+                lib.come_attn_set_exact_scale(1)
             _lib = lib
     return _lib
 

@@ -25,6 +25,7 @@
 //   the segment get scores of -inf and probabilities of exactly 0.
 #include "come_common.h"
 
+#include <atomic>
 #include <mutex>
 
 // Work buffer of come_attn_varlen_fwd_static: pieces of the key-split tail (unnormalised outputs, reference
@@ -176,14 +177,16 @@ constexpr int kStages = 4;
 
 // Direct global -> LDS loads (lane l of the wavefront lands at lds_addr + 16 l, resp. + 4 l), written as
 // asm so that the compiler does not order them against LDS reads it cannot tell apart: completion is
-// awaited explicitly with s_waitcnt vmcnt before the barrier that publishes the tile.
+// awaited explicitly with s_waitcnt vmcnt before the barrier that publishes the tile.  m0 carries the LDS address;
+// it is a register the compiler reserves and never keeps a value in across statements (it cannot be named as a
+// clobber: the compiler rejects reserved registers there).
 __device__ inline void dma_b128(const char *base, uint32_t lane_offset, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :: "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory", "m0");
+                 :: "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory");
 }
 __device__ inline void dma_b32(const char *base, uint32_t lane_offset, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
-                 :: "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory", "m0");
+                 :: "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory");
 }
 __device__ inline uint32_t lds_address(const void *p) {
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void *)(p)));
@@ -193,16 +196,20 @@ __device__ inline uint32_t lds_address(const void *p) {
 //   kSumLimit  a half-tile row sum above this moves the reference point of the row up
 //   kMaxGap    a row whose own maximum lies further below the workgroup's reference point keeps its own offset
 template <int DT> struct Range;
+//   kHardLimit a half-tile row sum above this may come from probabilities that left the 16-bit type's range
+//              (infinite, or saturated): the workgroup then computes its block again with a running maximum
 template <> struct Range<COME_BF16> {
     static constexpr float kSumLimit = 1099511627776.f;   // 2^40
     static constexpr float kMaxGap = 64.f;
+    static constexpr float kHardLimit = 1e38f;             // anything finite is fine: bf16 has the exponent range of fp32
 };
 template <> struct Range<COME_F16> {
     static constexpr float kSumLimit = 32.f;               // 2^5: a probability may grow by 2^11 more before fp16 saturates
     static constexpr float kMaxGap = 4.f;
+    static constexpr float kHardLimit = 32768.f;           // one probability near 65504 (where the conversion saturates)
 };
 
-template <int DT, int NW>
+template <int DT, int NW, bool EXACT>
 __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a) {
     using E = Elem<DT>;
     constexpr float kSumLimit = Range<DT>::kSumLimit;
@@ -250,7 +257,9 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     const int r = lane & 31;
     constexpr float kLog2e = 1.4426950408889634f;
 
-    // ---- Q fragments (B operand: n = query r, k = head-dim 16 ks + 8 h ..), scaled by c
+    // ---- Q fragments (B operand: n = query r, k = head-dim 16 ks + 8 h ..).  Scaled by c here and rounded back to
+    // 16 bit; EXACT: left as they are - the scores leave the MFMA unscaled and c is applied in fp32 in front of the
+    // exponential, as the reference applies it (softmax.h:76-88).
     u32x4 qf[2][4];
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
@@ -259,10 +268,14 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             const u32x4 raw = *reinterpret_cast<const u32x4 *>(qp + 16 * ks);
+            if (EXACT) {
+                qf[qt][ks] = raw;
+            } else {
 #pragma unroll
-            for (int w = 0; w < 4; ++w)
-                qf[qt][ks][w] = E::pack2(E::to_f32(static_cast<uint16_t>(raw[w] & 0xffffu)) * a.scale_log2,
-                                         E::to_f32(static_cast<uint16_t>(raw[w] >> 16)) * a.scale_log2);
+                for (int w = 0; w < 4; ++w)
+                    qf[qt][ks][w] = E::pack2(E::to_f32(static_cast<uint16_t>(raw[w] & 0xffffu)) * a.scale_log2,
+                                             E::to_f32(static_cast<uint16_t>(raw[w] >> 16)) * a.scale_log2);
+            }
         }
     }
     // ---- global -> LDS staging.  Wavefront w fills rows 16 w .. 16 w + 15 of a tile with two direct
@@ -400,7 +413,8 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
         for (int ks = 0; ks < 4; ++ks) {
             const u32x4 kf = *reinterpret_cast<const u32x4 *>(&lds_k[buf][k_rd[ks] + 32 * half * kHeadDim]);
 #pragma unroll
-            for (int qt = 0; qt < 2; ++qt) s_acc[b][qt] = E::mfma(kf, qf[qt][ks], ks == 0 ? seed : s_acc[b][qt]);
+            for (int qt = 0; qt < 2; ++qt)
+                s_acc[b][qt] = E::mfma(kf, qf[qt][ks], ks == 0 ? (EXACT ? zero16 : seed) : s_acc[b][qt]);
         }
     };
     // O^T += V^T P^T of both query tiles for half-tile `half` of the V tile in `buf`, probabilities of buffer b
@@ -419,6 +433,16 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
         }
     };
 
+    // EXACT: bias log2(e) - m_base of the keys behind accumulator elements e, e + 1 (e even) of half-tile `half` in
+    // stage `buf`: not the initial value of the accumulator but added, together with the scale, in front of the
+    // exponential (one fused multiply-add per score)
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    const float c_scale = a.scale_log2;
+    const float inv_c = 1.0f / a.scale_log2;
+    auto seed_pair = [&](int buf, int half, int e) __attribute__((always_inline)) -> f32x2 {
+        return *reinterpret_cast<const f32x2 *>(&lds_b[buf][32 * half + 8 * (e >> 2) + b_rd + (e & 3)]);
+    };
+
     // One slot in explicit issue order.  The vector ALU turns the scores in buffer X (one 32-key half-tile,
     // both query tiles) into probabilities.  Meanwhile the matrix pipe builds the scores of the next
     // half-tile in buffer Y (8 MFMAs on 4 K fragments, each fragment shared by both query tiles) and
@@ -427,12 +451,19 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     // fragments (four MFMAs) ahead, so an in-order wavefront always has independent work behind each
     // MFMA.  sched_barrier keeps the compiler from regrouping the chunks.
     // Returns through sum[qt] the row sums of this lane over the half-tile.
-    auto slot = [&](int X, int Y, int kbuf, int khalf, int vbuf, int vhalf, float (&sum)[2]) __attribute__((always_inline)) {
+    // (xbuf, xhalf): stage and half of the half-tile whose scores sit in buffer X (EXACT reads its seeds from there)
+    auto slot = [&](int X, int Y, int xbuf, int xhalf, int kbuf, int khalf, int vbuf, int vhalf, float (&sum)[2]) __attribute__((always_inline)) {
         // fragments 0..3: V (u, dt) of the P V MFMAs 0..7; fragments 4..7: K k-steps of the score MFMAs 8..15.
         // P V goes first: the probabilities of buffer Y die while those of buffer X are born, and the score
         // registers of buffer Y are not needed before half of buffer X has been consumed.
         u32x4 frag[8];
         f32x16 seed;                  // bias log2(e) - m_base of this lane's 16 keys of the half-tile being scored
+        f32x2 sd[8];                  // EXACT: seeds of the half-tile being exponentiated, read two chunks ahead
+        if (EXACT) {
+            seed = zero16;
+            sd[0] = seed_pair(xbuf, xhalf, 0);
+            sd[1] = seed_pair(xbuf, xhalf, 2);
+        }
         auto request = [&](int f) __attribute__((always_inline)) {
             if (f < 4) {
                 const int u = f >> 1, dt = f & 1;
@@ -466,7 +497,8 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
             // one MFMA per chunk: P V MFMAs 0..7, score MFMAs 8..15; fragments are requested four chunks ahead
             issue(c);
             if ((c & 1) == 0 && c <= 10) request((c >> 1) + 2);      // chunk 0 -> fragment 2, ..., chunk 10 -> fragment 7
-            if (c >= 1 && c <= 4) {                                  // initial values of the scores, needed by chunk 8
+            if (EXACT && c + 2 < 8) sd[c + 2] = seed_pair(xbuf, xhalf, 2 * (c + 2));   // (chunk c + 8 uses the pair of chunk c again)
+            if (!EXACT && c >= 1 && c <= 4) {                        // initial values of the scores, needed by chunk 8
                 const f32x4 bq = *reinterpret_cast<const f32x4 *>(&lds_b[kbuf][32 * khalf + 8 * (c - 1) + b_rd]);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) seed[4 * (c - 1) + e] = bq[e];
@@ -478,6 +510,10 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
                 sum[qt] = E::dot2_ones(pw, sum[qt]);
             }
             float s0 = s_acc[X][c >> 3][2 * (c & 7)], s1 = s_acc[X][c >> 3][2 * (c & 7) + 1];
+            if (EXACT) {
+                s0 = __builtin_fmaf(s0, c_scale, sd[c & 7][0]);
+                s1 = __builtin_fmaf(s1, c_scale, sd[c & 7][1]);
+            }
             p0 = __builtin_amdgcn_exp2f(s0);
             p1 = __builtin_amdgcn_exp2f(s1);
             asm volatile("" : "+v"(p0), "+v"(p1));
@@ -515,6 +551,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     //    which are relative to the old reference, have been accumulated.
     float o_pending[2] = {1.f, 1.f};
     bool any_pending = false;                  // wave-uniform
+    bool overflowed = false;                   // wave-uniform: some half-tile row sum exceeded kHardLimit
     auto finish_slot = [&](int Y, const float (&sum)[2]) __attribute__((always_inline)) {
         const bool bad = !(sum[0] <= kSumLimit) || !(sum[1] <= kSumLimit);
         if (__any(bad) || any_pending || has_delta) {
@@ -527,12 +564,13 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
                 if (any_pending) scale_o(qt, o_pending[qt]);
                 float row_sum = sum[qt];
                 asm volatile("" : "+v"(row_sum));       // keeps the arithmetic of this rare path inside the branch
+                overflowed = overflowed || __any(!(row_sum <= Range<DT>::kHardLimit));
                 int shift = row_sum <= kSumLimit ? 0 : max(__builtin_amdgcn_frexp_expf(row_sum) - 2, 1);
                 shift = static_cast<int>(max_across_halves(static_cast<float>(shift)));   // both half-waves of a row agree
                 const float down = __builtin_amdgcn_exp2f(static_cast<float>(-shift));
                 delta[qt] += static_cast<float>(shift);
                 m_run[qt] += static_cast<float>(shift);
-                const float d = delta[qt];
+                const float d = EXACT ? delta[qt] * inv_c : delta[qt];       // EXACT: the accumulators hold unscaled scores
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     float t = s_acc[Y][qt][e];
@@ -588,9 +626,18 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     float wave_max = -INFINITY;
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
-        float mx = s_acc[0][qt][0];
+        float mx = -INFINITY;
+        if (EXACT) {
 #pragma unroll
-        for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s_acc[0][qt][e]);
+            for (int e = 0; e < 16; e += 2) {
+                const f32x2 sd = seed_pair(0, 0, e);
+                mx = fmaxf(mx, fmaxf(__builtin_fmaf(s_acc[0][qt][e], c_scale, sd[0]),
+                                     __builtin_fmaf(s_acc[0][qt][e + 1], c_scale, sd[1])));
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[0][qt][e]);
+        }
         mx = max_across_halves(mx);
         row_max[qt] = (mx == -INFINITY || mx != mx) ? 0.f : mx;
         wave_max = fmaxf(wave_max, row_max[qt]);
@@ -611,49 +658,121 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
         const float gap = row_max[qt] - m_base;
         delta[qt] = gap < -Range<DT>::kMaxGap ? floorf(gap) : 0.f;
         m_run[qt] = m_base + delta[qt];
+        // the same scores, now relative to the reference (EXACT: m_base reaches them through the seeds in LDS)
+        const float back = EXACT ? delta[qt] * inv_c : m_run[qt];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s_acc[0][qt][e] -= m_run[qt];     // the same scores, now relative to the reference
+        for (int e = 0; e < 16; ++e) s_acc[0][qt][e] -= back;
     }
     has_delta = __any(delta[0] != 0.f || delta[1] != 0.f);
     __syncthreads();                   // the rebased bias values are visible
 
     // A wavefront whose 64 queries all lie beyond the end of the segment (last workgroup of a segment) only
     // helps with the staging: it has nothing to compute and nothing to write.  Wavefront 0 always has queries.
-    if (q0 + wave_u * 64 >= L) {
+    const bool idle = q0 + wave_u * 64 >= L;
+    if (idle) {
         for (int j = 0; j < n_tiles; ++j) {
             stage_k(j + 3, (j + 3) & 3);
             stage_v(j + 2, (j + 2) & 3);
             staged_wait(true);
             __syncthreads();
         }
-        return;
+    } else {
+        for (int j = 0; j < n_tiles; ++j) {
+            const int kb = j & 3, kb1 = (j + 1) & 3, kb2 = (j + 2) & 3, kb3 = (j + 3) & 3;   // stage of tile j, j+1, ..
+            load_bias(j + 4, kb);      // raw bias runs one more tile ahead (converted between the slots of iteration j+2)
+            stage_k(j + 3, kb3);       // K(j+3) replaces K(j-1), V(j+2) replaces V(j-2): both idle since the
+            stage_v(j + 2, kb2);       // last barrier; they are first read two barriers from now
+            float sum[2];
+            peek_bias(kb2);
+            // slot a: keys 0..31 of tile j become probabilities; scores of keys 32..63; P V of keys 32..63 of tile j-1
+            slot(0, 1, kb, 0, kb, 1, kb3, 1, sum);
+            finish_slot(1, sum);
+            commit_bias(j + 2, kb2);   // raw bias landed before the last barrier; published by the next one
+            // slot b: keys 32..63 of tile j become probabilities; scores of keys 0..31 of tile j+1; P V of keys 0..31 of tile j
+            slot(1, 0, kb, 1, kb1, 0, kb, 0, sum);
+            finish_slot(0, sum);
+
+            staged_wait(true);         // loads issued one iteration ago have landed
+            __syncthreads();
+        }
+        pv_mfma(1, (n_tiles - 1) & 3, 1);      // keys 32..63 of the last tile
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o_acc[qt][dt][e] *= o_pending[qt];
     }
 
-    for (int j = 0; j < n_tiles; ++j) {
-        const int kb = j & 3, kb1 = (j + 1) & 3, kb2 = (j + 2) & 3, kb3 = (j + 3) & 3;   // stage of tile j, j+1, ..
-        load_bias(j + 4, kb);          // raw bias runs one more tile ahead (converted between the slots of iteration j+2)
-        stage_k(j + 3, kb3);           // K(j+3) replaces K(j-1), V(j+2) replaces V(j-2): both idle since the
-        stage_v(j + 2, kb2);           // last barrier; they are first read two barriers from now
-        float sum[2];
-        peek_bias(kb2);
-        // slot a: keys 0..31 of tile j become probabilities; scores of keys 32..63; P V of keys 32..63 of tile j-1
-        slot(0, 1, kb, 1, kb3, 1, sum);
-        finish_slot(1, sum);
-        commit_bias(j + 2, kb2);       // raw bias landed before the last barrier; published by the next one
-        // slot b: keys 32..63 of tile j become probabilities; scores of keys 0..31 of tile j+1; P V of keys 0..31 of tile j
-        slot(1, 0, kb1, 0, kb, 0, sum);
-        finish_slot(0, sum);
-
-        staged_wait(true);             // loads issued one iteration ago have landed
-        __syncthreads();
+    // ---- Probabilities are stored in the 16-bit type relative to a reference point that follows the scores lazily.
+    // A key that beats everything its row has seen by more than that type can hold (2^127 for bf16, about 2^15 for
+    // fp16) within one 32-key step leaves an infinite or saturated probability behind.  The wavefront that saw such a
+    // row sum says so here, and the workgroup then computes its block once more with the textbook running maximum
+    // (one tile at a time, no pipelining: slow, exact for any scores, and never taken by ordinary attention logits).
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // no direct load is in flight any more
+    if (lane == 0) lds_ref[wave] = overflowed ? 1.f : 0.f;
+    __syncthreads();
+    bool again = false;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) again = again || lds_ref[w] != 0.f;
+    if (again) {
+        m_base = 0.f;                                           // the seeds are absolute now
+        float m_row[2] = {-INFINITY, -INFINITY};
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+            o_acc[qt][0] = zero16;
+            o_acc[qt][1] = zero16;
+            l_run[qt] = 0.f;
+        }
+        for (int j = 0; j < n_tiles; ++j) {
+            __syncthreads();                                    // stage 0 is free again
+            load_bias(j, 0);
+            stage_k(j, 0);
+            stage_v(j, 0);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            peek_bias(0);
+            commit_bias(j, 0);
+            __syncthreads();
+            if (idle) continue;
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                score_mfma(0, 0, half);
+#pragma unroll
+                for (int qt = 0; qt < 2; ++qt) {
+                    float ex[16];
+                    float mx = -INFINITY;
+#pragma unroll
+                    for (int e = 0; e < 16; e += 2) {
+                        const f32x2 sd = seed_pair(0, half, e);
+                        ex[e] = EXACT ? __builtin_fmaf(s_acc[0][qt][e], c_scale, sd[0]) : s_acc[0][qt][e];
+                        ex[e + 1] = EXACT ? __builtin_fmaf(s_acc[0][qt][e + 1], c_scale, sd[1]) : s_acc[0][qt][e + 1];
+                        mx = fmaxf(mx, fmaxf(ex[e], ex[e + 1]));
+                    }
+                    mx = fmaxf(max_across_halves(mx), m_row[qt]);
+                    const float ref = mx == -INFINITY ? 0.f : mx;          // a row that has seen masked keys only
+                    const float down = __builtin_amdgcn_exp2f(m_row[qt] - ref);
+                    m_row[qt] = mx;
+#pragma unroll
+                    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) o_acc[qt][dt][e] *= down;
+                    float part = 0.f;
+#pragma unroll
+                    for (int w = 0; w < 8; ++w) {
+                        const uint32_t pw = E::pack2_prob(__builtin_amdgcn_exp2f(ex[2 * w] - ref),
+                                                          __builtin_amdgcn_exp2f(ex[2 * w + 1] - ref));
+                        p_frag[0][qt][w >> 2][w & 3] = pw;
+                        part = E::dot2_ones(pw, part);
+                    }
+                    l_run[qt] = l_run[qt] * down + part;
+                }
+                pv_mfma(0, 0, half);
+            }
+        }
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) m_run[qt] = m_row[qt] == -INFINITY ? 0.f : m_row[qt];
     }
-    pv_mfma(1, (n_tiles - 1) & 3, 1);      // keys 32..63 of the last tile
-#pragma unroll
-    for (int qt = 0; qt < 2; ++qt)
-#pragma unroll
-        for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) o_acc[qt][dt][e] *= o_pending[qt];
+    if (idle) return;
 
     // ---- epilogue of a split workgroup: unnormalised outputs, reference point and row sum of its key share
     if (piece != nullptr) {
@@ -825,6 +944,11 @@ extern "C" int64_t come_attn_work_bytes(int64_t n_seq, int64_t total, int64_t n_
     return make_plan(n_seq, total, n_heads, max_seqlen, true).work_bytes;
 }
 
+// Process-wide: apply softmax_scale in fp32 behind the score MFMA instead of folding it into a 16-bit Q.
+static std::atomic<int> g_exact_scale{0};
+
+extern "C" int come_attn_set_exact_scale(int on) { return g_exact_scale.exchange(on != 0 ? 1 : 0); }
+
 // Address of this device's copy of `scratch` (nullptr + error message on failure).  The array's name is only a
 // host-side handle: the device address is asked for once per device, with that device current, and kept.
 static void *static_work_pointer() {
@@ -931,13 +1055,20 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
                  "come_attn_varlen_fwd: grid too large");
     const dim3 grid(static_cast<unsigned>(n_wg)), block(wide ? 512 : 256);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool exact = g_exact_scale.load(std::memory_order_relaxed) != 0;
+#define COME_ATTN_LAUNCH(DT_, NW_)                                                                              \
+    do {                                                                                                        \
+        if (exact) hipLaunchKernelGGL((attn_fwd_pipe_kernel<DT_, NW_, true>), grid, block, 0, s, a);            \
+        else hipLaunchKernelGGL((attn_fwd_pipe_kernel<DT_, NW_, false>), grid, block, 0, s, a);                 \
+    } while (0)
     if (wide) {
-        if (dtype == COME_BF16) hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_BF16, 8>), grid, block, 0, s, a);
-        else hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_F16, 8>), grid, block, 0, s, a);
+        if (dtype == COME_BF16) COME_ATTN_LAUNCH(COME_BF16, 8);
+        else COME_ATTN_LAUNCH(COME_F16, 8);
     } else {
-        if (dtype == COME_BF16) hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_BF16, 4>), grid, block, 0, s, a);
-        else hipLaunchKernelGGL((attn_fwd_pipe_kernel<COME_F16, 4>), grid, block, 0, s, a);
+        if (dtype == COME_BF16) COME_ATTN_LAUNCH(COME_BF16, 4);
+        else COME_ATTN_LAUNCH(COME_F16, 4);
     }
+#undef COME_ATTN_LAUNCH
     COME_CHECK_LAUNCH("come_attn_varlen_fwd");
     if (plan.splits > 1) {
         static_assert(kHeadDim / 4 == 16, "a workgroup of the combine kernel covers 16 rows of 16 four-element chunks");

@@ -15,7 +15,17 @@ __all__ = [
     "flash_attn_varlen_qkvpacked_func",
     "flash_attn_varlen_qkvpacked_func_w_perkey_bias",
     "infer_flash_attn_varlen_max_seqlen",
+    "set_exact_softmax_scale",
 ]
+
+
+def set_exact_softmax_scale(on: bool) -> bool:
+    """Process-wide: apply ``softmax_scale`` in fp32 to every score (as the reference's kernel does) instead of folding
+    it into a 16-bit Q.  About 10 % slower; for logits of tens of nats (large q / k norm gains).  Returns the previous
+    setting.  The environment variable ``COME_ATTN_EXACT_SCALE=1`` switches it on when the library is loaded."""
+    from ... import _lib
+
+    return bool(_lib.load().come_attn_set_exact_scale(1 if on else 0))
 
 
 def infer_flash_attn_varlen_max_seqlen(cu_seqlens: torch.Tensor) -> int:

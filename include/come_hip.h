@@ -195,10 +195,10 @@ int come_select_plan(const void *conf, int dtype, int64_t batch, int64_t frames,
  *   out       [total, n_heads, head_dim] of `dtype`, strides in elements
  *   lse       [n_heads, total] float: logsumexp of the biased, scaled scores (within 1e-2: the
  *             scaled q is rounded to 16 bits); may be NULL
- * Only head_dim == 64 is implemented.  Probabilities are kept relative to a lazily moved reference point of
- * their row and stored in `dtype`: with COME_BF16 a key may exceed everything its row has seen so far by 2^87
- * within one 32-key step, with COME_F16 only by about 2^11 (7.6 nats) before the stored probability saturates at 65504 (the result
- * stays finite but that key is under-weighted).
+ * Only head_dim == 64 is implemented.  Probabilities are kept relative to a lazily moved reference point of their
+ * row and stored in `dtype`; a workgroup that meets a key beating everything its rows have seen by more than that
+ * type can hold within one 32-key step (2^127 for COME_BF16, about 2^15 for COME_F16) computes its query block again
+ * with a running maximum, so the result is right for any finite scores.
  *
  * Stands in for varlen_fwd / varlen_fwd_w_perkey_bias
  * (src/cuda_extension/flash_attn/flash_api.cpp:291-607; kernel
@@ -215,6 +215,17 @@ int come_attn_varlen_fwd(const void *q, const void *k, const void *v, int dtype,
                          const void *perkey_bias, int64_t max_seqlen, float softmax_scale,
                          void *out, int64_t o_row_stride, int64_t o_head_stride,
                          float *lse, void *stream);
+
+/*
+ * come_attn_set_exact_scale — process-wide switch for how softmax_scale reaches the scores; returns the previous
+ * setting.
+ *   0 (default)  Q is multiplied by softmax_scale * log2(e) once and rounded back to `dtype`: a logit moves by up to
+ *                2^-9 of its size, which is inside the stated tolerance (1e-2 max-abs) for logits up to some ten nats;
+ *   1            Q enters the MFMA as it is and the scale is applied in fp32 to every score, as the reference applies
+ *                it (src/cuda_extension/flash_attn/src/softmax.h:76-88): one more vector instruction per score,
+ *                about 10 % slower, for callers whose logits reach tens of nats (large q / k norm gains).
+ */
+int come_attn_set_exact_scale(int on);
 
 /*
  * come_attn_varlen_fwd_ws — the same operator with a caller-supplied work buffer.  When the launch would end

@@ -18,7 +18,7 @@ from come_amd.cuda_extension import (
     flash_attn_varlen_qkvpacked_func_w_perkey_bias,
     infer_flash_attn_varlen_max_seqlen,
 )
-from come_amd.cuda_extension.flash_attn import flash_attn_fwd_cuda
+from come_amd.cuda_extension.flash_attn import flash_attn_fwd_cuda, set_exact_softmax_scale
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -26,6 +26,15 @@ MAX_ABS, MEAN_ABS = 1e-2, 1e-3
 
 SEGMENT_SETS = [[32, 48, 24, 24], [56, 49, 23], [128], [60, 40], [50], [128, 256], [100, 150, 50], [64] * 4,
                 [1], [3, 1, 2], [65], [257, 31], [700, 333, 64], [1000]]
+
+
+@pytest.fixture
+def exact_scale():
+    """Runs a test with softmax_scale applied in fp32 to every score (the reference's arithmetic) and restores the
+    default (scale folded into a 16-bit Q) afterwards."""
+    before = set_exact_softmax_scale(True)
+    yield
+    set_exact_softmax_scale(before)
 
 
 def _cu(lens):
@@ -120,6 +129,119 @@ def test_count_bias_equals_key_duplication():
     # log(9) rounded to bf16 is 2.203125 (exp -> 9.054): the identity holds to that rounding
     diff = (a.float() - b[:L].float()).abs()
     assert float(diff.max()) <= 2e-2 and float(diff.mean()) <= 2e-3
+
+
+def test_sharp_logits_with_exact_scale(exact_scale):
+    """The case that needs 8e-2 with the scale folded into a 16-bit Q (late_rows below: logits of up to +-35 nats
+    with near-ties between the leading keys) meets the ordinary tolerance when the scale is applied in fp32."""
+    L, H = 1500, 2
+    qkv = torch.randn(L, 3, H, 64).bfloat16()
+    qkv[:, 1, :, :] *= torch.linspace(0.2, 6.0, L)[:, None, None].bfloat16()
+    bias = torch.zeros(L).bfloat16()
+    cu = _cu([L])
+    ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias)
+    out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), L, perkey_bias=bias.to(DEV),
+                                                                 return_attn_probs=True)
+    diff = (out.float().cpu() - ref).abs()
+    torch.testing.assert_close(out.float().cpu(), ref, atol=1e-2, rtol=1e-2)
+    assert float(diff.mean()) <= MEAN_ABS
+    torch.testing.assert_close(lse.cpu(), ref_lse, atol=2e-3, rtol=1e-3)
+
+
+@pytest.mark.parametrize("gain", [1, 2, 4])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_layernormed_qk_with_gains_exact_scale(gain, dtype, exact_scale):
+    """What the real caller feeds the operator (reference vggt/module/bias_attention.py:100-137: q and k are
+    LayerNorm'd per head, so |q| = |k| = 8 * gain and logits reach 8 * gain^2 nats), at the ordinary tolerance."""
+    _check_layernormed(gain, dtype)
+
+
+def test_layernormed_qk_unit_gain_default_mode():
+    """With unit gains (logits within +-8 nats) the default mode - scale folded into a 16-bit Q - is inside the
+    tolerance as well; from a gain of 2 on it is not (measured max-abs 2.3e-2 at gain 2, 1.2e-1 at gain 4 in bf16),
+    which is what the exact mode is for."""
+    _check_layernormed(1, torch.bfloat16)
+    _check_layernormed(1, torch.float16)
+
+
+def _check_layernormed(gain, dtype):
+    lens, H = [700, 333, 64], 4
+    P = sum(lens)
+    g = torch.Generator().manual_seed(gain)
+    x = torch.randn(P, 3, H, 64, generator=g)
+    q = torch.nn.functional.layer_norm(x[:, 0], (64,)) * gain
+    k = torch.nn.functional.layer_norm(x[:, 1], (64,)) * gain
+    qkv = torch.stack((q, k, x[:, 2]), dim=1).to(dtype)
+    bias = torch.where(torch.rand(P, generator=g) < 0.3, math.log(9.0), 0.0).to(dtype)
+    cu = _cu(lens)
+    ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias)
+    out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), max(lens),
+                                                                 perkey_bias=bias.to(DEV), return_attn_probs=True)
+    diff = (out.float().cpu() - ref).abs()
+    torch.testing.assert_close(out.float().cpu(), ref, atol=1e-2, rtol=1e-2)
+    assert float(diff.mean()) <= MEAN_ABS
+    torch.testing.assert_close(lse.cpu(), ref_lse, atol=5e-3, rtol=1e-3)
+
+
+@pytest.mark.parametrize("mode", ["default", "exact"])
+@pytest.mark.parametrize("dtype,jump", [(torch.bfloat16, 100.0), (torch.bfloat16, 300.0), (torch.float16, 12.0),
+                                        (torch.float16, 30.0)], ids=["bf16+100", "bf16+300", "f16+12", "f16+30"])
+def test_late_key_beyond_the_range_of_the_stored_probabilities(dtype, jump, mode):
+    """A late key whose logit exceeds everything before it by `jump` nats: relative to the lazily moved reference
+    point its probability does not fit the 16-bit type (bf16: exp2 overflows from 88 nats on; fp16: the stored
+    value saturates from about 11 nats on).  The workgroup notices and computes its block again with a running
+    maximum, so the result meets the ordinary tolerance.  Several such keys, in the first tile, at tile borders and
+    in a second, short segment (tail block)."""
+    before = set_exact_softmax_scale(mode == "exact")
+    try:
+        lens, H = [1500, 90], 2
+        P = sum(lens)
+        g = torch.Generator().manual_seed(int(jump))
+        qkv = torch.randn(P, 3, H, 64, generator=g).to(dtype)
+        bias = torch.zeros(P)
+        bias[700] = jump                       # one step
+        bias[1023] = 2 * jump                  # a second one on top, last key of a tile
+        bias[1024] = 2 * jump - 1.0            # and a near-tie right behind it, first key of the next tile
+        bias[1500 + 40] = jump                 # second segment: inside its only query block
+        bias = bias.to(dtype)
+        assert bool(torch.isfinite(bias.float()).all())
+        cu = _cu(lens)
+        ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias)
+        out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), max(lens),
+                                                                     perkey_bias=bias.to(DEV), return_attn_probs=True)
+        assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(lse).all())
+        # two near-tied keys carry every row: the result is a 0.73 / 0.27 mix of two value rows, and rounding those
+        # two probabilities and the result to 16 bits alone costs about 2^-9 of the value (as in the reference's kernel)
+        diff = (out.float().cpu() - ref).abs()
+        torch.testing.assert_close(out.float().cpu(), ref, atol=1e-2, rtol=1e-2)     # the reference's own criterion
+        assert float(diff.mean()) <= MEAN_ABS + 2.0 ** -9 * float(ref.abs().mean()), f"mean-abs {float(diff.mean())}"
+        torch.testing.assert_close(lse.cpu(), ref_lse, atol=2e-2 if mode == "default" else 5e-3, rtol=1e-3)
+    finally:
+        set_exact_softmax_scale(before)
+
+
+def test_key_beyond_the_range_inside_a_key_split_piece():
+    """The same situation in a launch whose last query blocks are cut along the keys (long single segment with a work
+    buffer): the piece that meets the key computes its share again; pieces are combined as usual."""
+    L, H = 12288, 16
+    g = torch.Generator().manual_seed(9)
+    qkv = torch.randn(L, 3, H, 64, generator=g).bfloat16()
+    bias = torch.zeros(L)
+    bias[9000], bias[11500] = 120.0, 250.0
+    bias = bias.bfloat16()
+    from come_amd import _lib
+    assert _lib.load().come_attn_work_bytes(1, L, H, L) > 0
+    out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), _cu([L]).to(DEV), L,
+                                                                 perkey_bias=bias.to(DEV), return_attn_probs=True)
+    out, lse = out.float().cpu(), lse.cpu()
+    assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(lse).all())
+    q, k, v = qkv.float().unbind(1)
+    for row in [0, 255, 5000, 8999, 9000, 11776, 12000, 12287]:          # the last blocks are the split ones
+        scores = torch.einsum("hd,khd->hk", q[row], k) * 0.125 + bias.float()[None]
+        ref = torch.einsum("hk,khd->hd", torch.softmax(scores, -1), v)
+        diff = (out[row] - ref).abs()
+        assert float(diff.max()) <= MAX_ABS and float(diff.mean()) <= MEAN_ABS
+        torch.testing.assert_close(lse[:, row], torch.logsumexp(scores, -1), atol=2e-2, rtol=1e-3)
 
 
 @pytest.mark.parametrize("kind", ["ramp", "jump", "late_rows", "descending"])
