@@ -674,6 +674,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
             stage_k(j + 3, (j + 3) & 3);
             stage_v(j + 2, (j + 2) & 3);
             staged_wait(true);
+            if (lane == 0) lds_ref[wave] = 0.f;
             __syncthreads();
         }
     } else {
@@ -693,6 +694,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
             finish_slot(0, sum);
 
             staged_wait(true);         // loads issued one iteration ago have landed
+            if (lane == 0) lds_ref[wave] = overflowed ? 1.f : 0.f;      // (read behind the last of these barriers)
             __syncthreads();
         }
         pv_mfma(1, (n_tiles - 1) & 3, 1);      // keys 32..63 of the last tile
@@ -707,15 +709,13 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     // ---- Probabilities are stored in the 16-bit type relative to a reference point that follows the scores lazily.
     // A key that beats everything its row has seen by more than that type can hold (2^127 for bf16, about 2^15 for
     // fp16) within one 32-key step leaves an infinite or saturated probability behind.  The wavefront that saw such a
-    // row sum says so here, and the workgroup then computes its block once more with the textbook running maximum
+    // row sum said so in front of the loop's last barrier, and the workgroup then computes its block once more with the textbook running maximum
     // (one tile at a time, no pipelining: slow, exact for any scores, and never taken by ordinary attention logits).
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // no direct load is in flight any more
-    if (lane == 0) lds_ref[wave] = overflowed ? 1.f : 0.f;
-    __syncthreads();
     bool again = false;
 #pragma unroll
     for (int w = 0; w < NW; ++w) again = again || lds_ref[w] != 0.f;
     if (again) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // no direct load is in flight any more
         m_base = 0.f;                                           // the seeds are absolute now
         float m_row[2] = {-INFINITY, -INFINITY};
 #pragma unroll
