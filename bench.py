@@ -9,7 +9,7 @@ algorithmic flops (sum over segments of 4 L^2 d H) per second.
 
 The same line carries, under ``other``, the merge / unmerge microbenchmark (16 frames of 37x37,
 C = 1024, bf16, 3x3 windows, ratio 0.5) as GB/s of algorithmic bytes with its own roofline, and
-the select + plan + merge pipeline rate.
+the rate of the whole confidence-guided merge (selection + plan in one launch, then the gather-mean).
 
 ``roofline`` times the dominant kernel with HIP events on the launch stream; ``cpu_baseline`` times
 the reference's PyTorch CPU path (SDPA with the bias as attn_mask) on the same workload on the host
@@ -34,12 +34,14 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 
 # HBM bytes per launch of each kernel on exactly the workloads built below, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE passes (KiB per dispatch), FETCH_SIZE scaled by 2.000 and WRITE_SIZE by 1.000 -- the factors a 256 MiB
-# device copy (``--only copy``) gives for the same counters.  The summaries are in profiles/.
-TRAFFIC_BYTES = {
-    "attn": int((266700 * 2.000 + 97750) * 1024),
-    "merge": int((22070 * 2.000 + 25940) * 1024),
-    "unmerge": int((13570 * 2.000 + 43970) * 1024),
+# device copy (``--only copy``) gives for the same counters.  Each entry names the summary under profiles/ that holds
+# the run it was read from; a kernel change means a new run of the commands written there and new numbers here.
+TRAFFIC = {
+    "attn": {"bytes": int((266850 * 2.000 + 97745) * 1024), "source": "profiles/attn_fwd_c3.txt"},
+    "merge": {"bytes": int((22072 * 2.000 + 25943) * 1024), "source": "profiles/merge_c2_r050.txt"},
+    "unmerge": {"bytes": int((13632 * 2.000 + 43970) * 1024), "source": "profiles/unmerge_c2_r050.txt"},
 }
+TRAFFIC_BYTES = {k: v["bytes"] for k, v in TRAFFIC.items()}
 
 
 def parse_args():
@@ -50,7 +52,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "prologue", "copy", "e2e", "stress", "stress_e2e", "frame"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "prologue", "copy", "exact", "select", "e2e", "stress", "stress_e2e", "frame"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -252,15 +254,22 @@ def bench_merge_unmerge(device, iters=200, warmup=20):
                   "value": round(merge_gbs, 1), "unit": "GB/s", "us_per_call": round(merge_ms / iters * 1e3, 2),
                   "algorithmic_bytes": w["merge_bytes"], "iters": iters, "rotating_buffer_sets": len(w["outs"]),
                   "roofline": {"bound": "hbm", "achieved": round(merge_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                               "frac": round(merge_gbs / PEAK_HBM_GBS, 4), "traffic": TRAFFIC_BYTES["merge"]},
-                  "select_plan_merge_us": round(pipe_ms / iters * 1e3, 2),
+                               "frac": round(merge_gbs / PEAK_HBM_GBS, 4), "traffic": TRAFFIC_BYTES["merge"],
+                               "traffic_source": TRAFFIC["merge"]["source"]},
+                  # confidence -> mask -> plan (one launch, come_select_plan) -> gather-mean: the whole
+                  # confidence-guided merge, same algorithmic bytes (the selection reads the confidence map and
+                  # writes a few KB of bookkeeping, both already counted)
+                  "select_plan_merge": {"us_per_call": round(pipe_ms / iters * 1e3, 2),
+                                        "value": round(w["merge_bytes"] / (pipe_ms / iters * 1e-3) / 1e9, 1), "unit": "GB/s",
+                                        "frac": round(w["merge_bytes"] / (pipe_ms / iters * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
                   "select_plan_us": round(select_plan_ms / iters * 1e3, 2)},
         "unmerge": {"workload": "C2 unmerge: P=%d -> %d rows, C=1024 bf16" % (w["P"], w["frames"] * w["N"]),
                     "value": round(split_gbs, 1), "unit": "GB/s", "us_per_call": round(split_ms / iters * 1e3, 2),
                     "algorithmic_bytes": w["split_bytes"], "iters": iters, "rotating_buffer_sets": len(w["outs"]),
                     "roofline": {"bound": "hbm", "achieved": round(split_gbs, 1), "peak": PEAK_HBM_GBS,
                                  "unit": "GB/s", "frac": round(split_gbs / PEAK_HBM_GBS, 4),
-                                 "traffic": TRAFFIC_BYTES["unmerge"]}},
+                                 "traffic": TRAFFIC_BYTES["unmerge"],
+                                 "traffic_source": TRAFFIC["unmerge"]["source"]}},
     }
 
 
@@ -510,6 +519,29 @@ def bench_stress(device):
     return res
 
 
+def bench_exact_scale(device, steps=10, warmup=3):
+    """The headline workload with softmax_scale applied in fp32 to every score (``come_attn_set_exact_scale(1)``,
+    the reference's arithmetic) instead of folded into a 16-bit Q: what the optional mode costs."""
+    from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
+    from come_amd.cuda_extension.flash_attn import set_exact_softmax_scale
+
+    w = make_attention_workload(device)
+    max_len = max(w["lens"])
+
+    def step():
+        return flash_attn_varlen_qkvpacked_func_w_perkey_bias(w["qkv"], w["cu"], max_len, perkey_bias=w["bias"],
+                                                              softmax_scale=0.125)
+
+    before = set_exact_softmax_scale(True)
+    try:
+        _, ms = time_loop(step, steps, warmup)
+    finally:
+        set_exact_softmax_scale(before)
+    tflops = w["flops"] / (ms / steps * 1e-3) / 1e12
+    return {"ms_per_call": round(ms / steps, 4), "value": round(tflops, 1), "unit": "TFLOP/s",
+            "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
+
+
 def bench_gemm_reference(device):
     """Library bf16 GEMM (8192^3, N(0,1) operands, torch.matmul -> hipBLASLt) in the same run: what the matrix
     cores of this box sustain on data of the same kind, next to the nominal 2.5 PFLOP/s used for ``frac``."""
@@ -527,7 +559,9 @@ def bench_gemm_reference(device):
 def bench_e2e(device, frames=32, depth=24, reps=5, height=518, width=518, ratio=0.5):
     """End-to-end aggregator (random init, bf16): 24 frame + 24 global blocks, dim 1024, 16 heads x 64, MLP 4096,
     32 frames of 518x518; 3x3 merge from block 4 onward at ratio 0.5 against the same model without merging.
-    (``frames=128, width=392, ratio=0.75``: the long-sequence stress shape, 133 248 tokens.)"""
+    (``frames=128, depth=36, width=392, ratio=0.75``: the long-sequence stress configuration, 133 248 tokens.)
+    ``within_tolerance`` says whether the merged model stayed within the stated relative L1 of the unmerged one on
+    the pixels of unmerged windows; the same check is an assertion in tests/test_gpu_e2e_full.py."""
     import torch
     from come_amd.harness import AggregatorConfig, AlternatingAggregator, relative_l1
     from come_amd.token_merger import CoMe_2D_TokenMerger
@@ -557,13 +591,14 @@ def bench_e2e(device, frames=32, depth=24, reps=5, height=518, width=518, ratio=
     keep = torch.ones(frames, gh, gw, dtype=torch.bool, device=device)
     keep[:, :mh * 3, :mw * 3] = ~mask.repeat_interleave(3, 1).repeat_interleave(3, 2)
     keep_px = keep.repeat_interleave(14, 1).repeat_interleave(14, 2)[None, :, None]
+    rel = relative_l1(merged["maps"], dense["maps"], keep_px)
     return {"workload": f"VGGT-style aggregator, random init, bf16: {depth} frame + {depth} global blocks, dim 1024, "
                         f"16 heads x 64, MLP 4096, S={frames} frames {height}x{width} ({dense['tokens_dense']} tokens); "
                         f"3x3 merge from block {cfg.merge_block} at r={ratio} ({merged['tokens_packed']} packed tokens)",
             "merged_ms": round(merged_ms, 2), "unmerged_ms": round(dense_ms, 2),
             "speedup": round(dense_ms / merged_ms, 3), "reps": reps, "statistic": "median wall time per forward",
-            "rel_l1_unmerged_windows": round(relative_l1(merged["maps"], dense["maps"], keep_px), 5),
-            "rel_l1_tolerance": 5e-2}
+            "rel_l1_unmerged_windows": round(rel, 5), "rel_l1_tolerance": 5e-2, "within_tolerance": bool(rel <= 5e-2),
+            "finite": bool(torch.isfinite(merged["maps"]).all())}
 
 
 # ------------------------------------------------------------------------------------------
@@ -653,7 +688,7 @@ def main():
         elif args.only == "e2e":
             print(json.dumps({"only": "e2e", **bench_e2e(device, reps=max(1, args.steps))}))
         elif args.only == "stress_e2e":                          # seconds per forward: not part of the default run
-            print(json.dumps({"only": "stress_e2e", **bench_e2e(device, frames=128, width=392, ratio=0.75,
+            print(json.dumps({"only": "stress_e2e", **bench_e2e(device, frames=128, depth=36, width=392, ratio=0.75,
                                                                   reps=max(1, min(args.steps, 3)))}))
         elif args.only == "copy":
             # plain device copy of known size: the yardstick the HBM byte counters are scaled by
@@ -668,6 +703,8 @@ def main():
             w, wall, ev_ms = bench_attention(args.steps, args.warmup, device)
             print(json.dumps({"only": "attn", "ms_per_call": ev_ms / args.steps,
                               "tflops": w["flops"] / (ev_ms / args.steps * 1e-3) / 1e12}))
+        elif args.only == "exact":
+            print(json.dumps({"only": "exact", **bench_exact_scale(device, args.steps, args.warmup)}))
         elif args.only == "prologue":
             print(json.dumps({"only": "prologue", **bench_qk_prologue(device, iters=args.steps, warmup=args.warmup)}))
         elif args.only == "refmerge":
@@ -681,6 +718,10 @@ def main():
             for _ in range(len(mw["outs"])):
                 mw["merge_only"]()
             print(json.dumps({"only": "pair", **bench_unmerge_pair(device, mw, args.steps, args.warmup)}))
+        elif args.only == "select":
+            mw = merge_workload(device)
+            _, ms = time_loop(mw["select_and_plan"], args.steps, args.warmup)
+            print(json.dumps({"only": "select", "us_per_call": ms / args.steps * 1e3}))
         else:
             mw = merge_workload(device)
             for _ in range(len(mw["outs"])):
@@ -716,6 +757,7 @@ def main():
                    "algorithmic_flops_per_step": w["flops"]},
         "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(kernel_tflops / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES["attn"],
+                     "traffic_source": TRAFFIC["attn"]["source"],
                      "kernel": "attn_fwd_pipe_kernel<bf16>", "ms_per_launch": round(ev_ms / args.steps, 4)},
     }
     mw = None
@@ -730,6 +772,7 @@ def main():
         other["qk_prologue"] = bench_qk_prologue(device)
         other["frame_attention"] = bench_frame_attention(device, w)
         other["bias_overhead"] = bench_bias_overhead(device)
+        other["attention_exact_scale"] = bench_exact_scale(device)
         other["stress"] = bench_stress(device)
     if not args.no_e2e:
         result.setdefault("other", {})["e2e"] = bench_e2e(device)
