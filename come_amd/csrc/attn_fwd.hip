@@ -23,6 +23,12 @@
 //   (The reference adds bias / scale to the raw scores, flash_fwd_kernel.h:30-55, and
 //   subtracts the scaled running maximum inside exp2, softmax.h:76-88.)  Keys beyond the end of
 //   the segment get scores of -inf and probabilities of exactly 0.
+//   The reference point of a row moves lazily (only when a half-tile's row sum leaves the range the
+//   16-bit probabilities keep their precision in).  A workgroup in which a stored probability left
+//   the 16-bit range altogether raises a flag on the loop's last barrier and then computes its
+//   query block again, tile by tile, with a running maximum per row: any finite scores are exact.
+//   The EXACT instantiation keeps Q unscaled and applies c and the seed b_k - m_q per score in fp32
+//   (come_attn_set_exact_scale), for callers that want the reference's rounding of q k^T.
 #include "come_common.h"
 
 #include <atomic>

@@ -104,18 +104,37 @@ __device__ inline int leftover_position_fast(const MergeGeom &g, const FastDiv &
 }
 
 // ---------------------------------------------------------------------------------
-// bookkeeping: mask -> per-window prefix, per-row length, row offsets   (one workgroup)
+// bookkeeping: mask -> per-window prefix, per-row length, row offsets.  A wavefront owns a row; up to
+// kPlanRowsPerGroup rows run as one workgroup that also scans the lengths, more rows are spread
+// over workgroups and a one-wavefront launch scans afterwards.
 // ---------------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void merge_plan_kernel(const uint8_t *__restrict__ mask, int rows, int groups,
-                                                          int start, int G, int tail,
-                                                          int32_t *__restrict__ offsets,
-                                                          int32_t *__restrict__ prefix) {
+constexpr int kPlanRowsPerGroup = 16;
+
+__device__ inline void scan_row_lengths(int32_t *__restrict__ offsets, int rows) {   // one wavefront, in place
+    const int lane = threadIdx.x & 63;
+    int carry = 0;
+    for (int r0 = 0; r0 < rows; r0 += 64) {
+        const int r = r0 + lane;
+        int v = r < rows ? offsets[r + 1] : 0;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int t = __shfl_up(v, d);
+            if (lane >= d) v += t;
+        }
+        if (r < rows) offsets[r + 1] = v + carry;
+        carry += __shfl(v, 63);
+    }
+}
+
+__global__ __launch_bounds__(64 * kPlanRowsPerGroup) void merge_plan_kernel(const uint8_t *__restrict__ mask, int rows,
+                                                                            int groups, int start, int G, int tail,
+                                                                            int32_t *__restrict__ offsets,
+                                                                            int32_t *__restrict__ prefix) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int n_waves = blockDim.x >> 6;
     const uint64_t below = (1ull << lane) - 1ull;
 
-    for (int b = wave; b < rows; b += n_waves) {
+    for (int b = blockIdx.x * kPlanRowsPerGroup + wave; b < rows; b += gridDim.x * kPlanRowsPerGroup) {
         int running = 0;                                    // wave-uniform
         for (int m0 = 0; m0 < groups; m0 += 64) {
             const int m = m0 + lane;
@@ -130,23 +149,14 @@ __global__ __launch_bounds__(1024) void merge_plan_kernel(const uint8_t *__restr
         }
         if (lane == 0) offsets[b + 1] = start + tail + running;
     }
-    if (threadIdx.x == 0) offsets[0] = 0;
+    if (blockIdx.x == 0 && threadIdx.x == 0) offsets[0] = 0;
+    if (gridDim.x > 1) return;                              // the scan is the next launch
     __syncthreads();
+    if (wave == 0) scan_row_lengths(offsets, rows);
+}
 
-    if (wave == 0) {                                        // in-place inclusive scan of the row lengths
-        int carry = 0;
-        for (int r0 = 0; r0 < rows; r0 += 64) {
-            const int r = r0 + lane;
-            int v = r < rows ? offsets[r + 1] : 0;
-#pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                const int t = __shfl_up(v, d);
-                if (lane >= d) v += t;
-            }
-            if (r < rows) offsets[r + 1] = v + carry;
-            carry += __shfl(v, 63);
-        }
-    }
+__global__ __launch_bounds__(64) void merge_plan_scan_kernel(int32_t *__restrict__ offsets, int rows) {
+    scan_row_lengths(offsets, rows);
 }
 
 // ---------------------------------------------------------------------------------
@@ -507,9 +517,14 @@ extern "C" int come_merge_plan(const uint8_t *merge_mask, int64_t rows, int64_t 
     const int64_t n_tok = start_index + groups * group_size + tail;
     COME_REQUIRE(rows < (1ll << 31) && groups < (1ll << 31) && rows * n_tok < (1ll << 31), COME_ERR_UNSUPPORTED,
                  "come_merge_plan: rows * tokens per row must stay below 2^31");
-    hipLaunchKernelGGL(merge_plan_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream), merge_mask,
-                       static_cast<int>(rows), static_cast<int>(groups), static_cast<int>(start_index),
-                       static_cast<int>(group_size), static_cast<int>(tail), offsets, group_prefix);
+    const int plan_groups = static_cast<int>(std::min<int64_t>(std::max<int64_t>((rows + kPlanRowsPerGroup - 1) / kPlanRowsPerGroup, 1), 2048));
+    hipLaunchKernelGGL(merge_plan_kernel, dim3(plan_groups), dim3(64 * kPlanRowsPerGroup), 0,
+                       static_cast<hipStream_t>(stream), merge_mask, static_cast<int>(rows), static_cast<int>(groups),
+                       static_cast<int>(start_index), static_cast<int>(group_size), static_cast<int>(tail), offsets,
+                       group_prefix);
+    if (plan_groups > 1)
+        hipLaunchKernelGGL(merge_plan_scan_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), offsets,
+                           static_cast<int>(rows));
     COME_CHECK_LAUNCH("come_merge_plan");
     return COME_OK;
 }

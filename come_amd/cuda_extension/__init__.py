@@ -14,5 +14,3 @@ __all__ = [
     "flash_attn_varlen_qkvpacked_func_w_perkey_bias",
     "infer_flash_attn_varlen_max_seqlen",
 ]
-
-__version__ = "0.1.0"
