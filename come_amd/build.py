@@ -17,7 +17,7 @@ LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libcome_hip.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["abi.hip", "merge_kernels.hip", "select_kernels.hip", "attn_fwd.hip", "qk_prologue.hip", "suffix_kernels.hip"]
+SOURCES = ["abi.hip", "merge_kernels.hip", "select_kernels.hip", "attn_fwd.hip", "attn_fwd_hd.hip", "qk_prologue.hip", "suffix_kernels.hip"]
 
 # Packed-FP32 VALU forms are switched off for all device code.
 DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -29,7 +29,7 @@
 //   query block again, tile by tile, with a running maximum per row: any finite scores are exact.
 //   The EXACT instantiation keeps Q unscaled and applies c and the seed b_k - m_q per score in fp32
 //   (come_attn_set_exact_scale), for callers that want the reference's rounding of q k^T.
-#include "come_common.h"
+#include "attn_common.h"
 
 #include <atomic>
 #include <mutex>
@@ -42,97 +42,8 @@ static __device__ __align__(256) unsigned char scratch[kStaticWorkBytes];
 namespace come {
 namespace {
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-
 constexpr int kHeadDim = 64;
-constexpr int kBlockN = 64;          // keys per tile
-
-struct AttnArgs {
-    const uint16_t *q, *k, *v;
-    const uint16_t *bias;            // may be null
-    uint16_t *out;
-    float *lse;                      // may be null
-    const int32_t *cu;
-    int64_t q_rs, q_hs, k_rs, k_hs, v_rs, v_hs, o_rs, o_hs;
-    int64_t total;
-    int n_heads, n_mblocks, n_units;
-    float scale_log2;
-    // key-split tail: the last nb_tail query blocks of every (segment, head) unit are computed by `splits`
-    // workgroups each, every one over its share of the keys, into `work`; a second kernel combines them
-    int nb_tail, splits;
-    int64_t n_full_wg;               // workgroups in front of the split ones
-    float *work;
-};
-
 constexpr int kPieceExtra = 2;       // per query row of a piece: 64 unnormalised outputs, reference point, row sum
-
-
-template <int DT> struct Elem;
-template <> struct Elem<COME_BF16> {
-    static constexpr uint32_t kOne = 0x3F80u;
-    __device__ static inline float to_f32(uint16_t x) { return __uint_as_float(static_cast<uint32_t>(x) << 16); }
-    __device__ static inline uint16_t from_f32(float x) { return static_cast<uint16_t>(pack2_bf16(x, 0.f) & 0xffffu); }
-    __device__ static inline uint32_t pack2(float lo, float hi) { return pack2_bf16(lo, hi); }
-    __device__ static inline uint32_t pack2_prob(float lo, float hi) { return pack2_bf16(lo, hi); }
-    // acc + lo(w) + hi(w) with fp32 accumulation (v_dot2c_f32_bf16 against packed ones)
-    __device__ static inline float dot2_ones(uint32_t w, float acc) {
-        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(come_bf16x2, w),
-                                               __builtin_bit_cast(come_bf16x2, kOne | (kOne << 16)), acc, false);
-    }
-    __device__ static inline f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-    }
-};
-template <> struct Elem<COME_F16> {
-    static constexpr uint32_t kOne = 0x3C00u;
-    __device__ static inline float to_f32(uint16_t x) { return __half2float(__builtin_bit_cast(__half, x)); }
-    __device__ static inline uint16_t from_f32(float x) { return __builtin_bit_cast(uint16_t, __float2half_rn(x)); }
-    __device__ static inline uint32_t pack2(float lo, float hi) { return pack2_f16(lo, hi); }
-    // probabilities: round toward zero, so that a value beyond the fp16 range saturates at 65504 instead of
-    // becoming infinite (row sums are taken from the converted values, so numerator and denominator agree)
-    __device__ static inline uint32_t pack2_prob(float lo, float hi) {
-        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
-    }
-    __device__ static inline float dot2_ones(uint32_t w, float acc) {
-        return __builtin_amdgcn_fdot2(__builtin_bit_cast(come_f16x2, w),
-                                      __builtin_bit_cast(come_f16x2, kOne | (kOne << 16)), acc, false);
-    }
-    __device__ static inline f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-    }
-};
-
-__device__ inline u32x4 zero4() { return u32x4{0u, 0u, 0u, 0u}; }
-
-// exchange between lane l and lane l ^ 32: returns {value of the lower half lane, value of the upper half lane}
-__device__ inline float max_across_halves(float x) {
-    const uint32_t u = __float_as_uint(x);
-    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ inline float sum_across_halves(float x) {
-    const uint32_t u = __float_as_uint(x);
-    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-
-__device__ inline s16x4 lds_read_tr(const uint16_t *p) {
-    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(p));
-}
-
-// Offsets come from device memory that the host cannot check: a segment is clamped into [0, total], so that
-// inconsistent offsets give wrong results for their rows instead of accesses outside the tensors.
-__device__ inline void segment_of(const AttnArgs &a, int seq, int &seq_start, int &L) {
-    const int total = static_cast<int>(a.total);
-    seq_start = min(max(a.cu[seq], 0), total);
-    L = min(max(a.cu[seq + 1], seq_start), total) - seq_start;
-}
 
 // Which (segment, head, query block) a workgroup computes.  Workgroup i is dispatched to XCD
 // i % 8, each XCD with its own L2: the query blocks of one (segment, head) unit run back to back
@@ -181,22 +92,6 @@ __device__ inline bool locate_block(const AttnArgs &a, int &mblk, int &head, int
 // -------------------------------------------------------------------------------------
 constexpr int kStages = 4;
 
-// Direct global -> LDS loads (lane l of the wavefront lands at lds_addr + 16 l, resp. + 4 l), written as
-// asm so that the compiler does not order them against LDS reads it cannot tell apart: completion is
-// awaited explicitly with s_waitcnt vmcnt before the barrier that publishes the tile.  m0 carries the LDS address;
-// it is a register the compiler reserves and never keeps a value in across statements (it cannot be named as a
-// clobber: the compiler rejects reserved registers there).
-__device__ inline void dma_b128(const char *base, uint32_t lane_offset, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :: "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory");
-}
-__device__ inline void dma_b32(const char *base, uint32_t lane_offset, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
-                 :: "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory");
-}
-__device__ inline uint32_t lds_address(const void *p) {
-    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void *)(p)));
-}
 // Range of the probabilities relative to the reference point of their row.  They are stored in the 16-bit type of
 // the inputs: bf16 has the exponent range of fp32, fp16 reaches only 65504 and loses precision below 2^-14.
 //   kSumLimit  a half-tile row sum above this moves the reference point of the row up
@@ -992,8 +887,8 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
     clear_error();
     COME_REQUIRE(dtype == COME_BF16 || dtype == COME_F16, COME_ERR_UNSUPPORTED,
                  "come_attn_varlen_fwd: only fp16 and bf16 are supported");
-    COME_REQUIRE(head_dim == kHeadDim, COME_ERR_UNSUPPORTED,
-                 "come_attn_varlen_fwd: only head_dim == 64 is implemented (got %lld)", (long long)head_dim);
+    COME_REQUIRE(head_dim == 32 || head_dim == kHeadDim || head_dim == 128, COME_ERR_UNSUPPORTED,
+                 "come_attn_varlen_fwd: head_dim must be 32, 64 or 128 (got %lld)", (long long)head_dim);
     COME_REQUIRE(n_seq > 0, COME_ERR_INVALID, "come_attn_varlen_fwd: batch size must be positive");
     COME_REQUIRE(total >= 0 && n_heads > 0 && max_seqlen >= 0, COME_ERR_INVALID,
                  "come_attn_varlen_fwd: negative size");
@@ -1009,7 +904,7 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
     const int64_t strides[8] = {q_row_stride, q_head_stride, k_row_stride, k_head_stride,
                                 v_row_stride, v_head_stride, o_row_stride, o_head_stride};
     for (int i = 0; i < 8; ++i)
-        COME_REQUIRE(strides[i] >= kHeadDim || (i % 2 == 1 && n_heads == 1), COME_ERR_INVALID,
+        COME_REQUIRE(strides[i] >= head_dim || (i % 2 == 1 && n_heads == 1), COME_ERR_INVALID,
                      "come_attn_varlen_fwd: stride %d is smaller than head_dim", i);
     for (int i = 0; i < 6; ++i)
         COME_REQUIRE(strides[i] % 8 == 0, COME_ERR_UNSUPPORTED,
@@ -1020,6 +915,26 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
                      (reinterpret_cast<uintptr_t>(v) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0,
                  COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: q/k/v must be 16-byte aligned, out 8-byte aligned");
 
+    if (head_dim != kHeadDim) {               // the other widths: one kernel, no work buffer
+        AttnArgs a{};
+        a.q = static_cast<const uint16_t *>(q);
+        a.k = static_cast<const uint16_t *>(k);
+        a.v = static_cast<const uint16_t *>(v);
+        a.bias = static_cast<const uint16_t *>(perkey_bias);
+        a.out = static_cast<uint16_t *>(out);
+        a.lse = lse;
+        a.cu = cu_seqlens;
+        a.q_rs = q_row_stride; a.q_hs = q_head_stride;
+        a.k_rs = k_row_stride; a.k_hs = k_head_stride;
+        a.v_rs = v_row_stride; a.v_hs = v_head_stride;
+        a.o_rs = o_row_stride; a.o_hs = o_head_stride;
+        a.total = total;
+        a.n_heads = static_cast<int>(n_heads);
+        a.n_units = static_cast<int>(n_seq * n_heads);
+        a.scale_log2 = softmax_scale * 1.4426950408889634f;
+        a.splits = 1;
+        return launch_attn_hd(a, dtype, static_cast<int>(head_dim), max_seqlen, static_cast<hipStream_t>(stream));
+    }
     Plan plan = make_plan(n_seq, total, n_heads, max_seqlen, work != nullptr || static_work);
     if (static_work && plan.splits > 1) {
         COME_REQUIRE(plan.work_bytes <= kStaticWorkBytes, COME_ERR_UNSUPPORTED,

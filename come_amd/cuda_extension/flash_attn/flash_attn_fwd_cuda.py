@@ -101,8 +101,9 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
     _check(tuple(v.shape) == (total_k, num_heads_k, head_size), "v must have shape (total_k, num_heads_k, head_size)")
     _check(tuple(cu_seqlens_k.shape) == (batch_size + 1,), "cu_seqlens_k must have shape (batch_size + 1)")
     _unsupported(num_heads != num_heads_k, "grouped-query attention (num_heads != num_heads_k)")
-    if head_size > 64:
-        _unsupported(True, f"head_dim {head_size} (64 and, zero-padded, smaller multiples of 8 are implemented)")
+    if head_size > 128:
+        _unsupported(True, f"head_dim {head_size} (32, 64, 128 and, zero-padded, other multiples of 8 up to 128 "
+                           "are implemented)")
     _unsupported(total_q != total_k or max_seqlen_q != max_seqlen_k
                  or (cu_seqlens_q.data_ptr() != cu_seqlens_k.data_ptr() and not torch.equal(cu_seqlens_q, cu_seqlens_k)),
                  "cross attention (different query and key packing)")
@@ -119,11 +120,13 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
     def _aligned(t):          # the kernel issues 16-byte loads
         return t.data_ptr() % 16 == 0 and t.stride(0) % 8 == 0 and t.stride(1) % 8 == 0
 
-    if head_size < 64:
-        # narrower heads run on the 64-wide kernel: zero columns change neither q . k nor the other columns of
-        # the output (softmax_scale was fixed by the caller from the real width); costs a padded copy of q, k, v
-        padded = _varlen_fwd_impl(*(torch.nn.functional.pad(t, [0, 64 - head_size]) for t in (q, k, v)), None,
-                                  cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
+    kernel_width = 32 if head_size <= 32 else 64 if head_size <= 64 else 128
+    if head_size != kernel_width:
+        # in-between widths run zero-padded on the next kernel width: zero columns change neither q . k nor the
+        # other columns of the output (softmax_scale was fixed by the caller from the real width); costs a padded
+        # copy of q, k, v
+        padded = _varlen_fwd_impl(*(torch.nn.functional.pad(t, [0, kernel_width - head_size]) for t in (q, k, v)),
+                                  None, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
                                   perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, False, is_causal,
                                   window_size_left, window_size_right, softcap, return_softmax, gen)
         narrow = padded[0][..., :head_size]
@@ -155,7 +158,8 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
         if max_seqlen_k > 0:
             lib = _lib.load()
             # work buffer for the key-split tail of long launches (0 bytes: the launch does not use one)
-            work_bytes = lib.come_attn_work_bytes(batch_size, total_q, num_heads, max_seqlen_k)
+            work_bytes = (lib.come_attn_work_bytes(batch_size, total_q, num_heads, max_seqlen_k)
+                          if head_size == 64 else 0)
             work = torch.empty(work_bytes, dtype=torch.uint8, device=dev) if work_bytes > 0 else None
             _lib.check(lib.come_attn_varlen_fwd_ws(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.dtype_code(q.dtype),

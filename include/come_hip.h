@@ -195,10 +195,15 @@ int come_select_plan(const void *conf, int dtype, int64_t batch, int64_t frames,
  *   out       [total, n_heads, head_dim] of `dtype`, strides in elements
  *   lse       [n_heads, total] float: logsumexp of the biased, scaled scores (within 1e-2: the
  *             scaled q is rounded to 16 bits); may be NULL
- * Only head_dim == 64 is implemented.  Probabilities are kept relative to a lazily moved reference point of their
- * row and stored in `dtype`; a workgroup that meets a key beating everything its rows have seen by more than that
- * type can hold within one 32-key step (2^127 for COME_BF16, about 2^15 for COME_F16) computes its query block again
- * with a running maximum, so the result is right for any finite scores.
+ * head_dim is 32, 64 or 128 (the reference instantiates 32 ... 256 in steps of 32,
+ * src/cuda_extension/flash_attn/src/flash_fwd_launch_template.h:174-330; callers pad other widths up to 128 with
+ * zero columns, which changes neither q . k nor the other output columns).
+ * head_dim 64, the width of the shipped models: probabilities are kept relative to a lazily moved reference point
+ * of their row and stored in `dtype`; a workgroup that meets a key beating everything its rows have seen by more than
+ * that type can hold within one 32-key step (2^127 for COME_BF16, about 2^15 for COME_F16) computes its query block
+ * again with a running maximum, so the result is right for any finite scores.
+ * head_dim 32 and 128: one 32-query tile per wavefront, scale and bias applied to the fp32 scores (as with
+ * come_attn_set_exact_scale(1)), running maximum per row; no work buffer is used.
  *
  * Stands in for varlen_fwd / varlen_fwd_w_perkey_bias
  * (src/cuda_extension/flash_attn/flash_api.cpp:291-607; kernel

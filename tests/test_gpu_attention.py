@@ -362,7 +362,7 @@ def test_unsupported_arguments_raise():
     with pytest.raises(RuntimeError, match="dropout"):
         flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, 64, perkey_bias=bias, dropout_p=0.1)
     with pytest.raises(RuntimeError, match="head_dim"):
-        flash_attn_varlen_qkvpacked_func(torch.randn(P, 3, 2, 128, device=DEV).half(), cu, 64)
+        flash_attn_varlen_qkvpacked_func(torch.randn(P, 3, 2, 136, device=DEV).half(), cu, 64)
     with pytest.raises(RuntimeError, match="dtype"):
         flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, 64, perkey_bias=bias.half())
     with pytest.raises(RuntimeError, match="shape"):
@@ -487,8 +487,7 @@ def test_bias_of_minus_infinity_masks_keys():
 
 @pytest.mark.parametrize("lens", [[32, 48, 24, 24], [56, 49, 23], [128], [60, 40]], ids=str)
 def test_reference_test_shapes_with_narrow_heads(lens):
-    """The reference's own CUDA tests use heads of 32 (test_flex_attention_bias.py:247-262: H=2, D=32): they run
-    on the 64-wide kernel through zero padding."""
+    """The reference's own CUDA tests use heads of 32 (test_flex_attention_bias.py:247-262: H=2, D=32)."""
     P, H, D = sum(lens), 2, 32
     g = torch.Generator().manual_seed(P)
     qkv = torch.randn(P, 3, H, D, generator=g).bfloat16()
@@ -505,5 +504,5 @@ def test_reference_test_shapes_with_narrow_heads(lens):
         ref = torch.einsum("hqk,khd->qhd", torch.softmax(scores, -1), v[sl])
         torch.testing.assert_close(out[sl].float().cpu(), ref, atol=1e-2, rtol=1e-2)
         start += L
-    with pytest.raises(RuntimeError, match="head_dim 128"):
-        flash_attn_varlen_qkvpacked_func(torch.zeros(8, 3, 2, 128, device=DEV).bfloat16(), _cu([8]).to(DEV), 8)
+    with pytest.raises(RuntimeError, match="head_dim 256"):
+        flash_attn_varlen_qkvpacked_func(torch.zeros(8, 3, 2, 256, device=DEV).bfloat16(), _cu([8]).to(DEV), 8)
