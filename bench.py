@@ -52,7 +52,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "prologue", "copy", "exact", "select", "e2e", "stress", "stress_e2e", "frame"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "prologue", "copy", "exact", "widths", "select", "e2e", "stress", "stress_e2e", "frame"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -542,6 +542,31 @@ def bench_exact_scale(device, steps=10, warmup=3):
             "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
 
 
+def bench_other_widths(device, steps=10, warmup=3):
+    """The biased varlen attention at the head dimensions beside 64 that have their own kernel instance (32 and 128):
+    one segment of 16 384 tokens, 16 heads, bf16, bias log(count) on 30 % of the keys."""
+    import torch
+    from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
+
+    res = {}
+    L, H = 16384, 16
+    for D in (32, 128):
+        g = torch.Generator(device="cpu").manual_seed(D)
+        qkv = torch.randn(L, 3, H, D, generator=g).bfloat16().to(device)
+        bias = torch.where(torch.rand(L, generator=g) < 0.3, math.log(9.0), 0.0).bfloat16().to(device)
+        cu = torch.tensor([0, L], dtype=torch.int32, device=device)
+
+        def step():
+            return flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, L, perkey_bias=bias)
+
+        _, ms = time_loop(step, steps, warmup)
+        tflops = 4.0 * L * L * D * H / (ms / steps * 1e-3) / 1e12
+        res[f"head_dim_{D}"] = {"ms_per_call": round(ms / steps, 4), "value": round(tflops, 1), "unit": "TFLOP/s",
+                                "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
+    res["workload"] = "1 segment x 16384 tokens, 16 heads, bf16, per-key bias"
+    return res
+
+
 def bench_gemm_reference(device):
     """Library bf16 GEMM (8192^3, N(0,1) operands, torch.matmul -> hipBLASLt) in the same run: what the matrix
     cores of this box sustain on data of the same kind, next to the nominal 2.5 PFLOP/s used for ``frac``."""
@@ -705,6 +730,8 @@ def main():
                               "tflops": w["flops"] / (ev_ms / args.steps * 1e-3) / 1e12}))
         elif args.only == "exact":
             print(json.dumps({"only": "exact", **bench_exact_scale(device, args.steps, args.warmup)}))
+        elif args.only == "widths":
+            print(json.dumps({"only": "widths", **bench_other_widths(device, args.steps, args.warmup)}))
         elif args.only == "prologue":
             print(json.dumps({"only": "prologue", **bench_qk_prologue(device, iters=args.steps, warmup=args.warmup)}))
         elif args.only == "refmerge":
@@ -773,6 +800,7 @@ def main():
         other["frame_attention"] = bench_frame_attention(device, w)
         other["bias_overhead"] = bench_bias_overhead(device)
         other["attention_exact_scale"] = bench_exact_scale(device)
+        other["attention_other_widths"] = bench_other_widths(device)
         other["stress"] = bench_stress(device)
     if not args.no_e2e:
         result.setdefault("other", {})["e2e"] = bench_e2e(device)
