@@ -119,6 +119,18 @@ template <> struct Vec16<COME_F16> {
     }
 };
 
+// 16-byte global accesses; the streamed variants carry the non-temporal hint (data used once)
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ inline uint4 ld16(const uint4 *p) { return *p; }
+__device__ inline uint4 ld16_stream(const uint4 *p) {
+    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ inline void st16_stream(uint4 *p, const uint4 &v) {
+    const u32x4_t w = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(w, reinterpret_cast<u32x4_t *>(p));
+}
+
 inline int dtype_bytes(int dtype) { return dtype == COME_F32 ? 4 : 2; }
 inline bool dtype_ok(int dtype) { return dtype == COME_F32 || dtype == COME_F16 || dtype == COME_BF16; }
 

@@ -17,18 +17,6 @@ constexpr int kThreads = 256;
 // 16-frame microbenchmark: 14.2 / 14.6 / 14.8 / 16.0 / 18.1 us)
 constexpr int kMergeThreads = 64;
 
-// 16-byte global accesses; the streamed variants carry the non-temporal hint (data used once)
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-__device__ inline uint4 ld16(const uint4 *p) { return *p; }
-__device__ inline uint4 ld16_stream(const uint4 *p) {
-    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
-    return make_uint4(v[0], v[1], v[2], v[3]);
-}
-__device__ inline void st16_stream(uint4 *p, const uint4 &v) {
-    const u32x4_t w = {v.x, v.y, v.z, v.w};
-    __builtin_nontemporal_store(w, reinterpret_cast<u32x4_t *>(p));
-}
-
 // x / d for 0 <= x < 2^31 as one 32 x 32 -> 64 bit multiply and a shift (mul = ceil(2^shift / d),
 // shift = 31 + ceil(log2 d)); the index arithmetic of the 16-byte kernels runs on these instead of the
 // compiler's division sequences, which sit in front of every thread's first load

@@ -11,6 +11,9 @@
 //
 // Rounding follows a chain of tensor operations in the storage dtype: the normalised value
 // is rounded once, each of the two products is rounded, and their sum is rounded.
+//
+// The pass is bound by its in-place access pattern (4 KiB read and written out of every 6 KiB row of
+// the packed projection), not by arithmetic: loads and stores carry the non-temporal hint.
 #include "come_common.h"
 
 namespace come {
@@ -61,31 +64,67 @@ __device__ inline float group8_sum(float v) {
 
 constexpr int kRowsPerThread = 4;      // consecutive rows per lane: their loads are in flight together
 
+// Packed 16-bit pairs of the storage dtype: sum of a pair, and "first + sign * second", both in fp32 with one
+// rounding (a dot product against packed constants: the products with +-1 are exact).
+template <int DT> struct Pair;
+template <> struct Pair<COME_BF16> {
+    static constexpr uint32_t kOne = 0x3F80u, kMinusOne = 0xBF80u;
+    __device__ static inline float dot(uint32_t w, uint32_t k, float acc) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(come_bf16x2, w), __builtin_bit_cast(come_bf16x2, k), acc, false);
+    }
+    // the same without an accumulator (written out: the compiler otherwise zeroes a register for the in-place form)
+    __device__ static inline float dot0(uint32_t w, uint32_t k) {
+        float d;
+        asm("v_dot2_f32_bf16 %0, %1, %2, 0" : "=v"(d) : "v"(w), "v"(k));
+        return d;
+    }
+    __device__ static inline uint32_t pack(float lo, float hi) { return pack2_bf16(lo, hi); }
+};
+template <> struct Pair<COME_F16> {
+    static constexpr uint32_t kOne = 0x3C00u, kMinusOne = 0xBC00u;
+    __device__ static inline float dot(uint32_t w, uint32_t k, float acc) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(come_f16x2, w), __builtin_bit_cast(come_f16x2, k), acc, false);
+    }
+    __device__ static inline float dot0(uint32_t w, uint32_t k) {
+        float d;
+        asm("v_dot2_f32_f16 %0, %1, %2, 0" : "=v"(d) : "v"(w), "v"(k));
+        return d;
+    }
+    __device__ static inline uint32_t pack(float lo, float hi) { return pack2_f16(lo, hi); }
+};
+
+// Grid: x = groups of kRowsPerThread tokens, y = 256-thread slices of the 2 (q, k) x n_heads x 8 lanes of a token.
 template <int DT>
 __global__ void __launch_bounds__(256) qk_norm_rope_kernel(const QkArgs a) {
     using V = Vec16<DT>;
-    const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    const int lane8 = static_cast<int>(gid & 7);
-    const int64_t unit = gid >> 3;
-    const int head = static_cast<int>(unit % a.n_heads);
-    const int which = static_cast<int>((unit / a.n_heads) & 1);
-    const int64_t token0 = unit / (2 * a.n_heads) * kRowsPerThread;
-    if (token0 >= a.total) return;      // the eight lanes of a head leave together
+    using W = Pair<DT>;
+    const int j = blockIdx.y * 256 + threadIdx.x;                 // (which, head, lane8) of this lane
+    const int per_tensor = a.n_heads * 8;
+    if (j >= 2 * per_tensor) return;                              // the eight lanes of a head leave together
+    const int which = j >= per_tensor ? 1 : 0;
+    const int head = (j - which * per_tensor) >> 3;
+    const int lane8 = j & 7;
+    const int64_t token0 = static_cast<int64_t>(blockIdx.x) * kRowsPerThread;
 
-    uint4 *p[kRowsPerThread];
+    char *row = static_cast<char *>(a.ptr[which]) +
+                (token0 * a.row_stride[which] + head * a.head_stride[which]) * V::ELEM_BYTES + lane8 * 16;
+    const int64_t row_bytes = a.row_stride[which] * V::ELEM_BYTES;
     uint4 raw[kRowsPerThread];
-    int64_t pos[kRowsPerThread];
+    int entry[kRowsPerThread];                                    // byte offset of this lane's 8 table values
     bool live[kRowsPerThread];
 #pragma unroll
     for (int t = 0; t < kRowsPerThread; ++t) {
         live[t] = token0 + t < a.total;
         const int64_t token = live[t] ? token0 + t : token0;
-        p[t] = reinterpret_cast<uint4 *>(static_cast<char *>(a.ptr[which]) +
-                                         (token * a.row_stride[which] + head * a.head_stride[which]) * V::ELEM_BYTES) +
-               lane8;
-        raw[t] = *p[t];
-        // lanes 0-3 hold the y half, lanes 4-7 the x half of a head
-        pos[t] = a.positions != nullptr ? a.positions[token * 2 + (lane8 >> 2)] : 0;
+        raw[t] = ld16_stream(reinterpret_cast<const uint4 *>(row + (live[t] ? t : 0) * row_bytes));   // read once, written once
+        entry[t] = 0;
+        if (a.positions != nullptr) {
+            // lanes 0-3 hold the y half, lanes 4-7 the x half of a head; lanes {0,1} and {2,3} of a half are
+            // rotation partners and read the same 16 angles, 8 each
+            const int64_t pos = a.positions[token * 2 + (lane8 >> 2)];
+            const int pc = pos < 0 ? 0 : (pos >= a.n_pos ? static_cast<int>(a.n_pos) - 1 : static_cast<int>(pos));
+            entry[t] = (pc * 16 + (lane8 & 1) * 8) * V::ELEM_BYTES;
+        }
     }
     float g[8], b[8];
     if (a.apply_norm) {
@@ -102,49 +141,46 @@ __global__ void __launch_bounds__(256) qk_norm_rope_kernel(const QkArgs a) {
             for (int i = 0; i < 8; ++i) b[i] = 0.f;
         }
     }
+    constexpr uint32_t kOnes = W::kOne | (W::kOne << 16);
+    // the rotated partner enters with sign -1 in the first half of each 32-element block
+    const uint32_t one_and_sign = W::kOne | (((lane8 & 2) ? W::kOne : W::kMinusOne) << 16);
 
 #pragma unroll
     for (int t = 0; t < kRowsPerThread; ++t) {
+        uint4 word = raw[t];
         float f[8];
-        V::unpack(raw[t], f);
         if (a.apply_norm) {
-            float s = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) s += f[i];
+            // mean from the packed words, then the usual two passes in registers
+            float s = W::dot0(word.x, kOnes);
+            s = W::dot(word.y, kOnes, s);
+            s = W::dot(word.z, kOnes, s);
+            s = W::dot(word.w, kOnes, s);
             const float mean = group8_sum(s) * (1.0f / 64.0f);
+            V::unpack(word, f);
             float q = 0.f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 f[i] -= mean;
-                q += f[i] * f[i];
+                q = fmaf(f[i], f[i], q);
             }
             const float rstd = rsqrtf(group8_sum(q) * (1.0f / 64.0f) + a.eps);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) f[i] = f[i] * rstd * g[i] + b[i];
-            round_to_dtype<DT>(f);
+            for (int i = 0; i < 8; ++i) f[i] = fmaf(f[i] * rstd, g[i], b[i]);
+            word = V::pack(f);                                   // the normalised value is rounded once
         }
         if (a.positions != nullptr) {
-            // lanes {0,1} and {2,3} of a half are rotation partners
-            int64_t pc = pos[t];
-            pc = pc < 0 ? 0 : (pc >= a.n_pos ? a.n_pos - 1 : pc);
-            const int64_t entry = (pc * 16 + (lane8 & 1) * 8) * V::ELEM_BYTES;
-            float c[8], sn[8], r[8];
-            V::unpack(*reinterpret_cast<const uint4 *>(static_cast<const char *>(a.cos_table) + entry), c);
-            V::unpack(*reinterpret_cast<const uint4 *>(static_cast<const char *>(a.sin_table) + entry), sn);
-            const float sign = (lane8 & 2) ? 1.f : -1.f;
+            V::unpack(word, f);
+            float c[8], sn[8];
+            V::unpack(*reinterpret_cast<const uint4 *>(static_cast<const char *>(a.cos_table) + entry[t]), c);
+            V::unpack(*reinterpret_cast<const uint4 *>(static_cast<const char *>(a.sin_table) + entry[t]), sn);
+            // x cos and partner sin are rounded as a pair; their signed sum is one dot product and is rounded by
+            // the final pack
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                r[i] = lane_move<kSwapQuadHalves>(f[i]) * sn[i];
-                f[i] = f[i] * c[i];
-            }
-            round_to_dtype<DT>(r);
-            round_to_dtype<DT>(f);
-            // the rotated partner enters with sign -1 in the first half of each 32-element block (rounding is
-            // symmetric, so the sign can wait until the sum)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) f[i] = fmaf(sign, r[i], f[i]);
+            for (int i = 0; i < 8; ++i)
+                f[i] = W::dot0(W::pack(f[i] * c[i], lane_move<kSwapQuadHalves>(f[i]) * sn[i]), one_and_sign);
+            word = V::pack(f);
         }
-        if (live[t]) *p[t] = V::pack(f);
+        if (live[t]) st16_stream(reinterpret_cast<uint4 *>(row + t * row_bytes), word);
     }
 }
 
@@ -198,14 +234,14 @@ extern "C" int come_qk_norm_rope(void *q, void *k, int dtype,
     a.cos_table = cos_table;
     a.sin_table = sin_table;
     a.n_pos = n_pos;
-    const int64_t threads = ceil_div(total, kRowsPerThread) * 2 * n_heads * 8;
-    const int64_t blocks = ceil_div(threads, 256);
-    COME_REQUIRE(blocks < (int64_t{1} << 31), COME_ERR_UNSUPPORTED, "come_qk_norm_rope: too many tokens for one launch");
+    const int64_t groups = ceil_div(total, kRowsPerThread);
+    const int64_t slices = ceil_div(2 * n_heads * 8, 256);
+    COME_REQUIRE(groups < (int64_t{1} << 31) && slices < 65536 && n_pos < (1 << 24), COME_ERR_UNSUPPORTED,
+                 "come_qk_norm_rope: too many tokens, heads or positions for one launch");
+    const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(slices));
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == COME_BF16)
-        hipLaunchKernelGGL((qk_norm_rope_kernel<COME_BF16>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, a);
-    else
-        hipLaunchKernelGGL((qk_norm_rope_kernel<COME_F16>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, a);
+    if (dtype == COME_BF16) hipLaunchKernelGGL((qk_norm_rope_kernel<COME_BF16>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((qk_norm_rope_kernel<COME_F16>), grid, dim3(256), 0, s, a);
     COME_CHECK_LAUNCH("come_qk_norm_rope");
     return COME_OK;
 }
