@@ -42,7 +42,7 @@ def test_version_and_error_string():
     assert lib.come_token_merge(None, 7, 1, 1, 1, 0, 1, 1, 1, 1, None, None, None, None, 0,
                                 None, None, None, None, None) == 2
     assert b"dtype" in lib.come_last_error()
-    assert lib.come_attn_varlen_fwd(None, None, None, _lib.COME_BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 128,
+    assert lib.come_attn_varlen_fwd(None, None, None, _lib.COME_BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 96,
                                     None, 10, 0.125, None, 64, 64, None, None) == 2
     assert b"head_dim" in lib.come_last_error()
     assert lib.come_select_work_bytes(1, 16, 37, 37, 3, 3) >= 16 * 144 * 4
