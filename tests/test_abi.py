@@ -109,7 +109,7 @@ def test_every_entry_point_rejects_bad_arguments_on_the_host():
                                       None, 10, -1.0, None, 64, 64, None, None), "softmax_scale")
     rejected(lib.come_attn_varlen_fwd(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 64,
                                       None, 10, 0.125, None, 64, 64, None, None), "NULL")
-    rejected(lib.come_attn_varlen_fwd_ws(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 32,
+    rejected(lib.come_attn_varlen_fwd_ws(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 48,
                                          None, 10, 0.125, None, 64, 64, None, None, 0, None), "head_dim")
     rejected(lib.come_qk_norm_rope(None, None, F32, 64, 64, 64, 64, 4, 1, 64, 1, None, None, None, None, 1e-5,
                                    None, None, None, 0, None), "bf16 or fp16")
