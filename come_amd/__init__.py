@@ -7,7 +7,7 @@ Three operators, all backed by hand-written HIP kernels in ``libcome_hip.so``
   window selection, gather-mean into packed tokens + index map + counts + offsets),
 * unmerge (gather back to the dense token grid),
 * forward attention over packed variable-length sequences with an additive
-  per-key bias (head_dim 64).
+  per-key bias (head_dim 64, the width of the shipped models; 32 and 128 as well).
 
 ``come_amd.cuda_extension`` mirrors the module layout and names of the
 reference's ``src/cuda_extension`` package so callers switch by changing one

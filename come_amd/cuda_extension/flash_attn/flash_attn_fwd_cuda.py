@@ -3,7 +3,8 @@
 Positional signatures and return lists follow the reference's pybind module
 ``flash_attn_fwd_cuda`` (``src/cuda_extension/flash_attn/flash_api.cpp:538-607``,
 checks ``:291-408``, bias checks ``:274-288``).  Only what the Co-Me call sites
-reach is implemented: fp16 / bf16, head_dim 64 (narrower heads are zero-padded to it), self-attention over one set of
+reach is implemented: fp16 / bf16, head_dim 32 / 64 / 128 (other multiples of 8 up to 128 are zero-padded to the next
+of them), self-attention over one set of
 ``cu_seqlens``, no causal mask, no dropout, no alibi / softcap / sliding window /
 paged KV / left padding.  Anything else raises ``RuntimeError`` instead of
 computing something different.
