@@ -200,3 +200,30 @@ def test_unsupported_width_is_rejected_by_the_library():
                                   out.stride(1), None, _lib.current_stream(torch.device(DEV)))
     assert rc == 2                                           # COME_ERR_UNSUPPORTED
     assert b"head_dim" in lib.come_last_error()
+
+
+@pytest.mark.parametrize("D,H", [(128, 8), (32, 16)])
+def test_long_packed_sequences_sampled_rows(D, H):
+    """Two packed sequences of 25 536 and 21 848 tokens (the lengths of the 64-wide benchmark workload), bias =
+    log(count): the full fp32 oracle is too slow on a CPU at this size, so a sample of query rows is checked
+    against the closed form, plus the logsumexp identity."""
+    lens = [25536, 21848]
+    P = sum(lens)
+    g = torch.Generator().manual_seed(D)
+    qkv = torch.randn(P, 3, H, D, generator=g).bfloat16()
+    count = torch.ones(P)
+    count[torch.randperm(P, generator=g)[:5000]] = 9.0
+    bias = count.log().bfloat16()
+    cu = _cu(lens)
+    out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), max(lens),
+                                                                 perkey_bias=bias.to(DEV), return_attn_probs=True)
+    out, lse = out.float().cpu(), lse.cpu()
+    assert bool(torch.isfinite(out).all())
+    q, k, v = qkv.float().unbind(1)
+    for row in [0, 31, 32, 127, 128, 12345, 25535, 25536, 25537, 30000, P - 1]:
+        s, e = (0, lens[0]) if row < lens[0] else (lens[0], P)
+        scores = torch.einsum("hd,khd->hk", q[row], k[s:e]) * D ** -0.5 + bias.float()[None, s:e]
+        ref = torch.einsum("hk,khd->hd", torch.softmax(scores, -1), v[s:e])
+        diff = (out[row] - ref).abs()
+        assert float(diff.max()) <= 1e-2 and float(diff.mean()) <= 1e-3
+        torch.testing.assert_close(lse[:, row], torch.logsumexp(scores, -1), atol=2e-3, rtol=1e-3)
