@@ -49,7 +49,7 @@ def prepare_packed_self_attention_qkv(qkv: torch.Tensor, q_norm, k_norm, rope, p
                                       run_dtype: torch.dtype, max_position: int | None = None) -> torch.Tensor:
     """Normalises the packed q and k (``qkv [P, 3, H, D]``) and applies the 2-D RoPE, in place.
 
-    ``rope`` is an object with ``base_frequency`` (or ``None``), ``pos [P, 2]`` / ``[1, P, 2]`` integer
+    ``rope`` is an object with ``base_frequency`` or ``base`` (or ``None``), ``pos [P, 2]`` / ``[1, P, 2]`` integer
     (y, x).  ``max_position`` (largest coordinate that can occur) avoids the device-to-host read of
     ``pos.max()`` that sizes the frequency tables.
     """
@@ -82,8 +82,16 @@ def prepare_packed_self_attention_qkv(qkv: torch.Tensor, q_norm, k_norm, rope, p
         if positions.shape[0] != P:
             raise RuntimeError(f"pos must hold one (y, x) pair per packed row ({P}), got {positions.shape[0]}")
         n_pos = (int(positions.max().item()) if max_position is None else int(max_position)) + 1 if P > 0 else 1
-        if not isinstance(rope, RotaryPositionEmbedding2D):      # any object with a base frequency (e.g. the reference's)
-            rope = _TABLES.setdefault(float(rope.base_frequency), RotaryPositionEmbedding2D(float(rope.base_frequency)))
+        if not isinstance(rope, RotaryPositionEmbedding2D):
+            # the reference's rope modules: RotaryPositionEmbedding2D of VGGT / DA3 (``base_frequency``,
+            # thirdparty/vggt/layers/rope.py:78-83) and RoPE2D of Pi3 (``base``, thirdparty/pi3/models/layers/pos_embed.py:114-118);
+            # both build the same tables and apply x cos + rotate_half(x) sin per coordinate half
+            base = getattr(rope, "base_frequency", None)
+            if base is None:
+                base = getattr(rope, "base", None)
+            if base is None:
+                raise RuntimeError(f"rope must carry its base frequency as base_frequency or base, got {type(rope).__name__}")
+            rope = _TABLES.setdefault(float(base), RotaryPositionEmbedding2D(float(base)))
         cos_t, sin_t = rope.tables(D, n_pos, dev, run_dtype)
     q, k = qkv[:, 0], qkv[:, 1]
     lib = _lib.load()

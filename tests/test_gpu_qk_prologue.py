@@ -7,6 +7,7 @@ atol = 1e-2, and mean-abs <= 1e-3 over the tensor.
 """
 
 import copy
+import types
 
 import pytest
 import torch
@@ -73,6 +74,12 @@ def test_norm_only_rope_only_and_max_position():
         # a [1, P, 2] position tensor (as the reference passes it) is accepted
         c = prepare_packed_self_attention_qkv(qkv.cuda(), ident, ident, rope, pos[None].cuda(), dtype)
         assert torch.equal(c, b)
+        # rope modules of the reference are recognised by their attribute: VGGT / DA3 `base_frequency`, Pi3 `base`
+        for foreign in (types.SimpleNamespace(base_frequency=100.0), types.SimpleNamespace(base=100.0, F0=1.0)):
+            d = prepare_packed_self_attention_qkv(qkv.cuda(), ident, ident, foreign, pos.cuda(), dtype)
+            assert torch.equal(d, b)
+        with pytest.raises(RuntimeError, match="base frequency"):
+            prepare_packed_self_attention_qkv(qkv.cuda(), ident, ident, object(), pos.cuda(), dtype)
 
 
 def test_strided_views_of_a_wider_buffer():
