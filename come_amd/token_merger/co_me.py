@@ -7,6 +7,7 @@
 
 from __future__ import annotations
 
+import inspect
 from typing import Any, Callable
 
 import torch
@@ -64,12 +65,32 @@ def func_token_split_pair(tokens_a: JaggedTokens, tokens_b: JaggedTokens, rev_id
     return restored.reshape(B * S, N, 2 * C)
 
 
+def run_predictor(predictor, feature: torch.Tensor) -> torch.Tensor:
+    """Confidence of ``feature [B, S, C, H, W]`` from a predictor, one scalar per patch.
+
+    A plain callable gets the channels-last bf16 feature; the reference's predictor modules take the shape as a
+    keyword as well (``forward(tokens, BPHWC)``, src/accelerate/common/confidence_predictor.py:21, 51) and are
+    called the way the reference calls them (co_me.py:50, co_me_2d.py:264-267)."""
+    B, S, C, H, W = feature.shape
+    tokens = feature.permute(0, 1, 3, 4, 2).bfloat16()
+    forward = getattr(predictor, "forward", predictor)
+    try:
+        wants_shape = "BPHWC" in inspect.signature(forward).parameters
+    except (TypeError, ValueError):
+        wants_shape = False
+    confidence = predictor(tokens, BPHWC=(B, S, H, W, C)) if wants_shape else predictor(tokens)
+    if confidence.numel() != B * S * H * W:
+        raise ValueError(f"the predictor must return one confidence per patch ({B * S * H * W}), "
+                         f"got a tensor of shape {tuple(confidence.shape)}")
+    return confidence
+
+
 class CoMe_TokenMerger(ITokenMerger):
     """Groups of ``group_size`` consecutive tokens (reference ``CoMe_TokenMerger``, co_me.py:20-105).
 
     The confidence predictor is outside this package: pass a callable
-    ``predictor(feature [B,S,H,W,C] bf16) -> confidence [B, S*H*W]`` or hand the confidence to
-    ``build_ctx`` directly.  ``conf_mode`` uses the reference's names.
+    ``predictor(feature [B,S,H,W,C] bf16) -> confidence [B, S*H*W]`` (the reference's predictor modules work
+    as they are) or hand the confidence to ``build_ctx`` directly.  ``conf_mode`` uses the reference's names.
     """
 
     def __init__(self, start_idx: int, group_size: int, threshold: float,
@@ -88,7 +109,7 @@ class CoMe_TokenMerger(ITokenMerger):
         if confidence is None:
             if self.predictor is None:
                 raise ValueError("build_ctx needs a confidence tensor or a predictor")
-            confidence = self.predictor(feature.permute(0, 1, 3, 4, 2).bfloat16())
+            confidence = run_predictor(self.predictor, feature)
         if self.conf_mode == "pairwise-rank" and not (0.0 <= self.threshold <= 1.0):
             raise ValueError(f"Ranking mode requires threshold in [0, 1], got {self.threshold}")
         # groups of G consecutive tokens are 1 x G windows of a 1 x (H*W) grid.  Scope of the statistics as in the

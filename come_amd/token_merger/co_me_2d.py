@@ -21,7 +21,7 @@ import torch
 
 from ..cuda_extension.co_me import co_me_cuext
 from ..interface import ITokenMerger, JaggedTokens
-from .co_me import func_token_split, func_token_split_pair
+from .co_me import func_token_split, func_token_split_pair, run_predictor
 
 
 def _validate_token_merge_2d_args(tokens, start_index, group_h, group_w, H, W, merge_mask,
@@ -90,7 +90,7 @@ class CoMe_2D_TokenMerger(ITokenMerger):
         if confidence is None:
             if self.predictor is None:
                 raise ValueError("build_ctx needs a confidence tensor or a predictor")
-            confidence = self.predictor(feature.permute(0, 1, 3, 4, 2).bfloat16())
+            confidence = run_predictor(self.predictor, feature)
         if self.conf_mode == "pairwise-rank" and not (0.0 <= self.threshold <= 1.0):
             raise ValueError(f"Ranking mode requires threshold in [0, 1], got {self.threshold}")
         mask = co_me_cuext.co_me_select_windows(confidence.reshape(B * S, H, W), B, self.group_h, self.group_w,

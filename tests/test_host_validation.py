@@ -55,3 +55,25 @@ def test_split_pair_and_legacy_entry_points_on_the_host():
         co_me_cuext.co_me_token_merge_cuda_legacy(0, a, a, None)
     with pytest.raises(RuntimeError, match="not provided"):
         co_me_cuext.co_me_token_merge_scan_legacy(0, 2, a)
+
+
+def test_predictor_adapter_calls_reference_style_modules_with_the_shape():
+    """The reference's predictor modules take ``BPHWC`` beside the tokens and return ``[B*S, H*W, 1]``
+    (confidence_predictor.py:21-29, 51-75); a plain callable gets the tokens only."""
+    from come_amd.token_merger.co_me import run_predictor
+
+    class ReferenceStyle(torch.nn.Module):
+        def forward(self, tokens, BPHWC):
+            B, P, H, W, C = BPHWC
+            assert tokens.shape == (B, P, H, W, C) and tokens.dtype == torch.bfloat16
+            return tokens.reshape(B * P, H * W, C).float().mean(-1, keepdim=True)
+
+    feature = torch.randn(2, 3, 8, 4, 5)                       # [B, S, C, H, W]
+    want = feature.bfloat16().float().mean(2).reshape(6, 20)
+    got = run_predictor(ReferenceStyle(), feature)
+    assert got.shape == (6, 20, 1)
+    torch.testing.assert_close(got.squeeze(-1), want, atol=1e-2, rtol=1e-2)
+    plain = run_predictor(lambda t: t.float().mean(-1), feature)
+    torch.testing.assert_close(plain.reshape(6, 20), want, atol=1e-2, rtol=1e-2)
+    with pytest.raises(ValueError, match="one confidence per patch"):
+        run_predictor(lambda t: t.float(), feature)
