@@ -15,6 +15,7 @@ struct AttnArgs {
     int64_t q_rs, q_hs, k_rs, k_hs, v_rs, v_hs, o_rs, o_hs;
     int64_t total;
     int n_heads, n_mblocks, n_units;
+    int rotate;                      // unit u starts its query blocks at position u (even block counts, see locate_block)
     float scale_log2;
     // key-split tail: the last nb_tail query blocks of every (segment, head) unit are computed by `splits`
     // workgroups each, every one over its share of the keys, into `work`; a second kernel combines them

@@ -52,8 +52,12 @@ __global__ __launch_bounds__(256) void attn_fwd_hd_kernel(const AttnArgs a) {
     // workgroup i runs on XCD i % 8: the query blocks of one (segment, head) unit stay on one XCD
     const int xcd = blockIdx.x & 7;
     const int local = blockIdx.x >> 3;
-    const int unit = xcd + 8 * (local / a.n_mblocks);
-    const int mblk = local % a.n_mblocks;
+    const int unit_on_xcd = local / a.n_mblocks;
+    const int unit = xcd + 8 * unit_on_xcd;
+    // the workgroups of an XCD go to its four shader engines in turn: with an even number of blocks per unit, unit u
+    // starts its blocks at position u, so that the empty last blocks of short segments do not keep landing on the
+    // same engines
+    const int mblk = a.rotate ? (local % a.n_mblocks + unit_on_xcd) % a.n_mblocks : local % a.n_mblocks;
     if (unit >= a.n_units) return;
     const int head = unit % a.n_heads;
     const int seq = unit / a.n_heads;
@@ -261,6 +265,7 @@ __global__ __launch_bounds__(256) void attn_fwd_hd_kernel(const AttnArgs a) {
 int launch_attn_hd(const AttnArgs &args, int dtype, int head_dim, int64_t max_seqlen, hipStream_t stream) {
     AttnArgs a = args;
     a.n_mblocks = static_cast<int>(ceil_div(max_seqlen, 128));
+    a.rotate = a.n_mblocks % 2 == 0 ? 1 : 0;
     const int64_t n_wg = ceil_div(a.n_units, 8) * 8 * a.n_mblocks;
     COME_REQUIRE(n_wg < (1ll << 31), COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: grid too large");
     const dim3 grid(static_cast<unsigned>(n_wg)), block(256);
