@@ -99,3 +99,27 @@ def test_max_seqlen_may_be_any_upper_bound(lens):
         # the launch plan (workgroup width, key-split tail) may differ with the bound: same products, other order
         torch.testing.assert_close(out.float(), exact.float(), atol=4e-3, rtol=2 ** -7)
         torch.testing.assert_close(lse, exact_lse, atol=2e-3, rtol=1e-4)
+
+
+@pytest.mark.parametrize("width", [64, 32, 128])
+def test_every_block_count_covers_every_query_block_once(width):
+    """The order in which a launch visits the query blocks of a unit depends on the parity of the block count
+    (``max_seqlen`` / block rows): whatever the bound, every block is computed exactly once and the bits are the
+    same.  Unit counts that are not multiples of 8 and a segment shorter than one block are included."""
+    lens = [300, 77, 812, 5, 640]
+    heads = 3
+    P = sum(lens)
+    g = torch.Generator().manual_seed(width)
+    qkv = torch.randn(P, 3, heads, width, generator=g).bfloat16().to(DEV)
+    bias = (torch.rand(P, generator=g) * 3).log().clamp(min=-4).bfloat16().to(DEV)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32).to(DEV)
+    tight, tight_lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, max(lens), perkey_bias=bias,
+                                                                        return_attn_probs=True)
+    rows = 256 if width == 64 else 128
+    for extra in range(1, 10):
+        out = torch.full_like(tight, float("nan"))
+        got, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, max(lens) + extra * rows,
+                                                                     perkey_bias=bias, return_attn_probs=True)
+        out.copy_(got)
+        assert torch.equal(out, tight), f"{extra} more block rows"
+        assert torch.equal(lse, tight_lse)
