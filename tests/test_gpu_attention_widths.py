@@ -90,6 +90,12 @@ def test_long_segments_many_heads_and_other_scale(D):
     _run([2048, 1111], H=2, D=D, lse=True, max_seqlen=5000)                  # max_seqlen is only an upper bound
 
 
+@pytest.mark.parametrize("D", [32, 128])
+def test_empty_segments_between_others(D):
+    _run([40, 0, 90, 0], H=2, D=D, bias_kind="counts", lse=True)
+    _run([0, 130], H=1, D=D, bias_kind=None)
+
+
 @pytest.mark.parametrize("D", [8, 16, 24, 40, 72, 96, 120])
 def test_widths_in_between_run_zero_padded(D):
     _run([56, 49, 23], H=2, D=D)
