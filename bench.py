@@ -52,7 +52,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "prologue", "copy", "exact", "widths", "select", "e2e", "stress", "stress_e2e", "frame"], default=None,
+    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "prologue", "copy", "exact", "folded", "widths", "select", "e2e", "stress", "stress_e2e", "frame"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -135,7 +135,9 @@ def time_loop(fn, steps, warmup):
     return wall, start.elapsed_time(stop)
 
 
-def bench_attention(steps, warmup, device):
+def bench_attention(steps, warmup, device, scale_mode="auto"):
+    """The headline: the operator as a caller without any knowledge of its logits calls it (``scale_mode="auto"`` on
+    a plain tensor: softmax_scale applied in fp32 to every score, the reference's arithmetic)."""
     from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
 
     w = make_attention_workload(device)
@@ -143,7 +145,7 @@ def bench_attention(steps, warmup, device):
 
     def step():
         return flash_attn_varlen_qkvpacked_func_w_perkey_bias(w["qkv"], w["cu"], max_len, perkey_bias=w["bias"],
-                                                              softmax_scale=0.125)
+                                                              softmax_scale=0.125, scale_mode=scale_mode)
 
     wall, ev_ms = time_loop(step, steps, warmup)
     return w, wall, ev_ms
@@ -391,7 +393,7 @@ def bench_merge_ratios(device, iters=200, warmup=20):
     return out
 
 
-def attention_case(device, lens, counts, steps, warmup, H=16, D=64):
+def attention_case(device, lens, counts, steps, warmup, H=16, D=64, scale_mode="auto"):
     """Times the biased attention on packed segments ``lens`` with per-key counts; returns (ms, TFLOP/s)."""
     import torch
     from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
@@ -406,7 +408,8 @@ def attention_case(device, lens, counts, steps, warmup, H=16, D=64):
     cu = torch.tensor(bounds, dtype=torch.int32, device=device)
     max_len = max(lens)
     _, ms = time_loop(lambda: flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, max_len, perkey_bias=bias,
-                                                                             softmax_scale=0.125), steps, warmup)
+                                                                             softmax_scale=0.125,
+                                                                             scale_mode=scale_mode), steps, warmup)
     flops = sum(4.0 * n * n * D * H for n in lens)
     return ms / steps, flops / (ms / steps * 1e-3) / 1e12, flops
 
@@ -486,9 +489,12 @@ def bench_frame_attention(device, w):
     # launches of 0.1 - 0.2 ms: the figure settles only after some tens of milliseconds under load (142 us with 10
     # warm-up launches, 119 us from about 200 on), hence the long warm-up
     ms, tflops, flops = attention_case(device, lens, counts, steps=200, warmup=300)
+    ms_f, tflops_f, _ = attention_case(device, lens, counts, steps=200, warmup=100, scale_mode="folded")
     return {"workload": "frame attention: 32 segments of %d..%d packed tokens (same tokens as the headline sequence 0)"
                         % (min(lens), max(lens)), "us_per_call": round(ms * 1e3, 1), "value": round(tflops, 1),
-            "unit": "TFLOP/s", "algorithmic_flops": flops, "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
+            "unit": "TFLOP/s", "algorithmic_flops": flops, "frac": round(tflops / PEAK_BF16_TFLOPS, 4),
+            "folded_scale": {"us_per_call": round(ms_f * 1e3, 1), "value": round(tflops_f, 1),
+                             "frac": round(tflops_f / PEAK_BF16_TFLOPS, 4)}}
 
 
 def bench_stress(device):
@@ -514,37 +520,31 @@ def bench_stress(device):
     del w
     torch.cuda.empty_cache()
     ms, tflops, flops = attention_case(device, frame_lens, counts, steps=200, warmup=300)
-    res["frame_attention"] = {"us_per_call": round(ms * 1e3, 1), "TFLOPs": round(tflops, 1), "algorithmic_flops": flops}
+    ms_f, tflops_f, _ = attention_case(device, frame_lens, counts, steps=200, warmup=100, scale_mode="folded")
+    res["frame_attention"] = {"us_per_call": round(ms * 1e3, 1), "TFLOPs": round(tflops, 1), "algorithmic_flops": flops,
+                              "frac": round(tflops / PEAK_BF16_TFLOPS, 4),
+                              "folded_scale": {"us_per_call": round(ms_f * 1e3, 1), "TFLOPs": round(tflops_f, 1),
+                                               "frac": round(tflops_f / PEAK_BF16_TFLOPS, 4)}}
     ms, tflops, flops = attention_case(device, [P], counts, steps=5, warmup=2)
     res["global_attention"] = {"ms_per_call": round(ms, 3), "TFLOPs": round(tflops, 1), "algorithmic_flops": flops,
                                "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
     return res
 
 
-def bench_exact_scale(device, steps=10, warmup=3):
-    """The headline workload with softmax_scale applied in fp32 to every score (``come_attn_set_exact_scale(1)``,
-    the reference's arithmetic) instead of folded into a 16-bit Q: what the optional mode costs."""
-    from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
-    from come_amd.cuda_extension.flash_attn import set_exact_softmax_scale
-
-    w = make_attention_workload(device)
-    max_len = max(w["lens"])
-
-    def step():
-        return flash_attn_varlen_qkvpacked_func_w_perkey_bias(w["qkv"], w["cu"], max_len, perkey_bias=w["bias"],
-                                                              softmax_scale=0.125)
-
-    before = set_exact_softmax_scale(True)
-    try:
-        _, ms = time_loop(step, steps, warmup)
-    finally:
-        set_exact_softmax_scale(before)
+def bench_scale_mode(device, mode, steps=10, warmup=3):
+    """The headline workload with the way softmax_scale reaches the scores named explicitly: ``"exact"`` (in fp32 on
+    every score, the reference's arithmetic and the default for a tensor without a known logit bound) or ``"folded"``
+    (multiplied into a 16-bit q once: what tensors with a small ``come_qk_bound`` get)."""
+    w, _, ms = bench_attention(steps, warmup, device, scale_mode=mode)
     tflops = w["flops"] / (ms / steps * 1e-3) / 1e12
     return {"ms_per_call": round(ms / steps, 4), "value": round(tflops, 1), "unit": "TFLOP/s",
-            "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
+            "frac": round(tflops / PEAK_BF16_TFLOPS, 4),
+            "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(tflops / PEAK_BF16_TFLOPS, 4),
+                         "kernel": "attn_fwd_pipe_kernel<bf16, 8, %s>" % ("true" if mode == "exact" else "false")}}
 
 
-def bench_other_widths(device, steps=10, warmup=3):
+def bench_other_widths(device, steps=20, warmup=40):
     """The biased varlen attention at the head dimensions beside 64 that have their own kernel instance (32 and 128):
     one segment of 16 384 tokens, 16 heads, bf16, bias log(count) on 30 % of the keys."""
     import torch
@@ -730,8 +730,8 @@ def main():
             w, wall, ev_ms = bench_attention(args.steps, args.warmup, device)
             print(json.dumps({"only": "attn", "ms_per_call": ev_ms / args.steps,
                               "tflops": w["flops"] / (ev_ms / args.steps * 1e-3) / 1e12}))
-        elif args.only == "exact":
-            print(json.dumps({"only": "exact", **bench_exact_scale(device, args.steps, args.warmup)}))
+        elif args.only in ("exact", "folded"):
+            print(json.dumps({"only": args.only, **bench_scale_mode(device, args.only, args.steps, args.warmup)}))
         elif args.only == "widths":
             print(json.dumps({"only": "widths", **bench_other_widths(device, args.steps, args.warmup)}))
         elif args.only == "prologue":
@@ -787,7 +787,8 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(kernel_tflops / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES["attn"],
                      "traffic_source": TRAFFIC["attn"]["source"],
-                     "kernel": "attn_fwd_pipe_kernel<bf16>", "ms_per_launch": round(ev_ms / args.steps, 4)},
+                     "kernel": "attn_fwd_pipe_kernel<bf16, 8, true>", "scale_mode": "auto -> exact (fp32 scale on every score)",
+                     "ms_per_launch": round(ev_ms / args.steps, 4)},
     }
     mw = None
     if not args.no_other:
@@ -801,7 +802,8 @@ def main():
         other["qk_prologue"] = bench_qk_prologue(device)
         other["frame_attention"] = bench_frame_attention(device, w)
         other["bias_overhead"] = bench_bias_overhead(device)
-        other["attention_exact_scale"] = bench_exact_scale(device)
+        other["attention_exact_scale"] = bench_scale_mode(device, "exact")
+        other["attention_folded_scale"] = bench_scale_mode(device, "folded")
         other["attention_other_widths"] = bench_other_widths(device)
         other["stress"] = bench_stress(device)
     if not args.no_e2e:

@@ -17,6 +17,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("COME_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libcome_hip.so")
 
 COME_F32, COME_F16, COME_BF16 = 0, 1, 2
+COME_ATTN_FOLD_SCALE = 1          # bit of the attention entry points' `flags`
 
 _DTYPE_CODE = {torch.float32: COME_F32, torch.float16: COME_F16, torch.bfloat16: COME_BF16}
 
@@ -41,16 +42,15 @@ SIGNATURES = {
     "come_select_work_bytes": (_i64, [_i64, _i64, _i64, _i64, _i64, _i64]),
     "come_attn_varlen_fwd": (_int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64,
                                     _ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _f32,
-                                    _ptr, _i64, _i64, _ptr, _ptr]),
+                                    _ptr, _i64, _i64, _ptr, _int, _ptr]),
     "come_attn_work_bytes": (_i64, [_i64, _i64, _i64, _i64]),
-    "come_attn_set_exact_scale": (_int, [_int]),
     "come_attn_varlen_fwd_ws": (_int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64,
                                        _ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _f32,
-                                       _ptr, _i64, _i64, _ptr, _ptr, _i64, _ptr]),
+                                       _ptr, _i64, _i64, _ptr, _ptr, _i64, _int, _ptr]),
     "come_attn_static_work_bytes": (_i64, []),
     "come_attn_varlen_fwd_static": (_int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64,
                                            _ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _f32,
-                                           _ptr, _i64, _i64, _ptr, _ptr]),
+                                           _ptr, _i64, _i64, _ptr, _int, _ptr]),
     "come_qk_norm_rope": (_int, [_ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                  _int, _ptr, _ptr, _ptr, _ptr, _f32, _ptr, _ptr, _ptr, _i64, _ptr]),
     "come_jagged_add_suffix": (_int, [_ptr, _ptr, _int, _i64, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr]),
@@ -79,8 +79,6 @@ def load() -> ctypes.CDLL:
                 fn = getattr(lib, name)
                 fn.restype = restype
                 fn.argtypes = argtypes
-            if os.environ.get("COME_ATTN_EXACT_SCALE", "0") not in ("", "0"):
-                lib.come_attn_set_exact_scale(1)
             _lib = lib
     return _lib
 

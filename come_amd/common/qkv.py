@@ -45,6 +45,24 @@ def _norm_params(norm):
     raise RuntimeError(f"q_norm / k_norm must be LayerNorm or Identity, got {type(norm).__name__}")
 
 
+_BOUND_CACHE: dict = {}
+
+
+def _norm_bound(weight, bias, head_dim: int, run_dtype) -> float:
+    """Upper bound of the Euclidean norm of a LayerNorm'd head: ``sqrt(D) max|gain| + |bias|_2`` (the normalised
+    vector has norm ``<= sqrt(D)``), with gain and bias as the kernel uses them (rounded to the run dtype).  One
+    device read per parameter version, cached."""
+    key = (None if weight is None else (weight.data_ptr(), weight._version),
+           None if bias is None else (bias.data_ptr(), bias._version), head_dim, run_dtype)
+    if key not in _BOUND_CACHE:
+        if len(_BOUND_CACHE) > 4096:
+            _BOUND_CACHE.clear()
+        gain = 1.0 if weight is None else float(weight.detach().to(run_dtype).float().abs().max())
+        shift = 0.0 if bias is None else float(bias.detach().to(run_dtype).float().norm())
+        _BOUND_CACHE[key] = head_dim ** 0.5 * gain + shift
+    return _BOUND_CACHE[key]
+
+
 def prepare_packed_self_attention_qkv(qkv: torch.Tensor, q_norm, k_norm, rope, pos: torch.Tensor | None,
                                       run_dtype: torch.dtype, max_position: int | None = None) -> torch.Tensor:
     """Normalises the packed q and k (``qkv [P, 3, H, D]``) and applies the 2-D RoPE, in place.
@@ -52,6 +70,10 @@ def prepare_packed_self_attention_qkv(qkv: torch.Tensor, q_norm, k_norm, rope, p
     ``rope`` is an object with ``base_frequency`` or ``base`` (or ``None``), ``pos [P, 2]`` / ``[1, P, 2]`` integer
     (y, x).  ``max_position`` (largest coordinate that can occur) avoids the device-to-host read of
     ``pos.max()`` that sizes the frequency tables.
+
+    When q and k are LayerNorm'd, the returned tensor carries ``come_qk_bound``: an upper bound of ``|q . k|`` over
+    all pairs, ``(sqrt(D) max|gain_q| + |bias_q|) (sqrt(D) max|gain_k| + |bias_k|)`` (the rotation keeps norms; 2 %
+    are added for its rounding).  The attention operators use it to choose how ``softmax_scale`` is applied.
     """
     if torch.is_grad_enabled() and qkv.requires_grad:
         raise RuntimeError("prepare_packed_self_attention_qkv is forward only (in place); run it under torch.no_grad()")
@@ -101,4 +123,9 @@ def prepare_packed_self_attention_qkv(qkv: torch.Tensor, q_norm, k_norm, rope, p
                                          1 if apply_q else 0, _lib.ptr(qw), _lib.ptr(qb), _lib.ptr(kw), _lib.ptr(kb),
                                          q_eps, _lib.ptr(positions), _lib.ptr(cos_t), _lib.ptr(sin_t), n_pos,
                                          _lib.current_stream(dev)))
+    if apply_q:
+        qkv.come_qk_bound = 1.02 * _norm_bound(q_norm.weight, q_norm.bias, D, run_dtype) * \
+            _norm_bound(k_norm.weight, k_norm.bias, D, run_dtype)
+    elif hasattr(qkv, "come_qk_bound"):
+        del qkv.come_qk_bound
     return qkv

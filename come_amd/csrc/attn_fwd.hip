@@ -27,11 +27,11 @@
 //   16-bit probabilities keep their precision in).  A workgroup in which a stored probability left
 //   the 16-bit range altogether raises a flag on the loop's last barrier and then computes its
 //   query block again, tile by tile, with a running maximum per row: any finite scores are exact.
-//   The EXACT instantiation keeps Q unscaled and applies c and the seed b_k - m_q per score in fp32
-//   (come_attn_set_exact_scale), for callers that want the reference's rounding of q k^T.
+//   That is the instantiation COME_ATTN_FOLD_SCALE selects.  The default one (EXACT) keeps Q as it is: the
+//   accumulator starts from (b_k - m_q) / c and every score is multiplied by c in fp32 in front of the exponential,
+//   which is the reference's arithmetic (bias / scale added to the raw scores, scale applied inside exp2).
 #include "attn_common.h"
 
-#include <atomic>
 #include <mutex>
 
 // Work buffer of come_attn_varlen_fwd_static: pieces of the key-split tail (unnormalised outputs, reference
@@ -109,7 +109,9 @@ template <int DT> struct Range;
 template <> struct Range<COME_BF16> {
     static constexpr float kSumLimit = 1099511627776.f;   // 2^40
     static constexpr float kMaxGap = 64.f;
-    static constexpr float kHardLimit = 1e38f;             // anything finite is fine: bf16 has the exponent range of fp32
+    // bf16 has the exponent range of fp32, but the fp32 outputs collect p * v over the 32 keys of a step: 2^100
+    // leaves 2^27 of headroom for |v| and the accumulation, and is still far above kSumLimit
+    static constexpr float kHardLimit = 1.2676506e30f;     // 2^100
 };
 template <> struct Range<COME_F16> {
     static constexpr float kSumLimit = 32.f;               // 2^5: a probability may grow by 2^11 more before fp16 saturates
@@ -165,9 +167,9 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     const int r = lane & 31;
     constexpr float kLog2e = 1.4426950408889634f;
 
-    // ---- Q fragments (B operand: n = query r, k = head-dim 16 ks + 8 h ..).  Scaled by c here and rounded back to
-    // 16 bit; EXACT: left as they are - the scores leave the MFMA unscaled and c is applied in fp32 in front of the
-    // exponential, as the reference applies it (softmax.h:76-88).
+    // ---- Q fragments (B operand: n = query r, k = head-dim 16 ks + 8 h ..).  EXACT: as they are - the scores leave
+    // the MFMA unscaled and c is applied in fp32 in front of the exponential, as the reference applies it
+    // (softmax.h:76-88).  Otherwise scaled by c here and rounded back to 16 bit.
     u32x4 qf[2][4];
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
@@ -246,7 +248,11 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     };
     // conversion of the raw bias of one tile, split in two so that the LDS read is in flight during a slot:
     // peek_bias() requests the word, commit_bias() writes bias log2(e) - m_base as a float, -inf beyond the segment
-    float m_base = 0.f;           // reference point shared by the rows of the workgroup (uniform)
+    // EXACT: what the accumulators hold is in units of the raw scores, 1 / c of the exponent of exp2
+    const float c_scale = a.scale_log2;
+    const float inv_c = 1.0f / a.scale_log2;
+    const float unit = EXACT ? inv_c : 1.f;
+    float m_base = 0.f;           // reference point shared by the rows of the workgroup (uniform), log2 units
     uint32_t b_word = 0;
     auto peek_bias = [&](int buf) __attribute__((always_inline)) {
         if (wave_u == 0 && b_seg) b_word = lds_braw[buf][lane];
@@ -259,7 +265,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
                 const uint32_t at = b_mis + 2u * static_cast<uint32_t>(min(key, L - 1));
                 bias = E::to_f32(static_cast<uint16_t>((at & 2u) ? (b_word >> 16) : (b_word & 0xffffu)));
             }
-            lds_b[buf][lane] = key < L ? bias * kLog2e - m_base : -INFINITY;
+            lds_b[buf][lane] = key < L ? (bias * kLog2e - m_base) * unit : -INFINITY;
         }
     };
     auto staged_wait = [&](bool with_bias_load) __attribute__((always_inline)) {
@@ -322,7 +328,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
             const u32x4 kf = *reinterpret_cast<const u32x4 *>(&lds_k[buf][k_rd[ks] + 32 * half * kHeadDim]);
 #pragma unroll
             for (int qt = 0; qt < 2; ++qt)
-                s_acc[b][qt] = E::mfma(kf, qf[qt][ks], ks == 0 ? (EXACT ? zero16 : seed) : s_acc[b][qt]);
+                s_acc[b][qt] = E::mfma(kf, qf[qt][ks], ks == 0 ? seed : s_acc[b][qt]);
         }
     };
     // O^T += V^T P^T of both query tiles for half-tile `half` of the V tile in `buf`, probabilities of buffer b
@@ -341,16 +347,6 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
         }
     };
 
-    // EXACT: bias log2(e) - m_base of the keys behind accumulator elements e, e + 1 (e even) of half-tile `half` in
-    // stage `buf`: not the initial value of the accumulator but added, together with the scale, in front of the
-    // exponential (one fused multiply-add per score)
-    typedef float f32x2 __attribute__((ext_vector_type(2)));
-    const float c_scale = a.scale_log2;
-    const float inv_c = 1.0f / a.scale_log2;
-    auto seed_pair = [&](int buf, int half, int e) __attribute__((always_inline)) -> f32x2 {
-        return *reinterpret_cast<const f32x2 *>(&lds_b[buf][32 * half + 8 * (e >> 2) + b_rd + (e & 3)]);
-    };
-
     // One slot in explicit issue order.  The vector ALU turns the scores in buffer X (one 32-key half-tile,
     // both query tiles) into probabilities.  Meanwhile the matrix pipe builds the scores of the next
     // half-tile in buffer Y (8 MFMAs on 4 K fragments, each fragment shared by both query tiles) and
@@ -359,19 +355,12 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     // fragments (four MFMAs) ahead, so an in-order wavefront always has independent work behind each
     // MFMA.  sched_barrier keeps the compiler from regrouping the chunks.
     // Returns through sum[qt] the row sums of this lane over the half-tile.
-    // (xbuf, xhalf): stage and half of the half-tile whose scores sit in buffer X (EXACT reads its seeds from there)
-    auto slot = [&](int X, int Y, int xbuf, int xhalf, int kbuf, int khalf, int vbuf, int vhalf, float (&sum)[2]) __attribute__((always_inline)) {
+    auto slot = [&](int X, int Y, int kbuf, int khalf, int vbuf, int vhalf, float (&sum)[2]) __attribute__((always_inline)) {
         // fragments 0..3: V (u, dt) of the P V MFMAs 0..7; fragments 4..7: K k-steps of the score MFMAs 8..15.
         // P V goes first: the probabilities of buffer Y die while those of buffer X are born, and the score
         // registers of buffer Y are not needed before half of buffer X has been consumed.
         u32x4 frag[8];
-        f32x16 seed;                  // bias log2(e) - m_base of this lane's 16 keys of the half-tile being scored
-        f32x2 sd[8];                  // EXACT: seeds of the half-tile being exponentiated, read two chunks ahead
-        if (EXACT) {
-            seed = zero16;
-            sd[0] = seed_pair(xbuf, xhalf, 0);
-            sd[1] = seed_pair(xbuf, xhalf, 2);
-        }
+        f32x16 seed;                  // (bias log2(e) - m_base) * unit of this lane's 16 keys of the half-tile being scored
         auto request = [&](int f) __attribute__((always_inline)) {
             if (f < 4) {
                 const int u = f >> 1, dt = f & 1;
@@ -405,8 +394,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
             // one MFMA per chunk: P V MFMAs 0..7, score MFMAs 8..15; fragments are requested four chunks ahead
             issue(c);
             if ((c & 1) == 0 && c <= 10) request((c >> 1) + 2);      // chunk 0 -> fragment 2, ..., chunk 10 -> fragment 7
-            if (EXACT && c + 2 < 8) sd[c + 2] = seed_pair(xbuf, xhalf, 2 * (c + 2));   // (chunk c + 8 uses the pair of chunk c again)
-            if (!EXACT && c >= 1 && c <= 4) {                        // initial values of the scores, needed by chunk 8
+            if (c >= 1 && c <= 4) {                                  // initial values of the scores, needed by chunk 8
                 const f32x4 bq = *reinterpret_cast<const f32x4 *>(&lds_b[kbuf][32 * khalf + 8 * (c - 1) + b_rd]);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) seed[4 * (c - 1) + e] = bq[e];
@@ -419,8 +407,8 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
             }
             float s0 = s_acc[X][c >> 3][2 * (c & 7)], s1 = s_acc[X][c >> 3][2 * (c & 7) + 1];
             if (EXACT) {
-                s0 = __builtin_fmaf(s0, c_scale, sd[c & 7][0]);
-                s1 = __builtin_fmaf(s1, c_scale, sd[c & 7][1]);
+                s0 *= c_scale;
+                s1 *= c_scale;
             }
             p0 = __builtin_amdgcn_exp2f(s0);
             p1 = __builtin_amdgcn_exp2f(s1);
@@ -535,18 +523,9 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
         float mx = -INFINITY;
-        if (EXACT) {
 #pragma unroll
-            for (int e = 0; e < 16; e += 2) {
-                const f32x2 sd = seed_pair(0, 0, e);
-                mx = fmaxf(mx, fmaxf(__builtin_fmaf(s_acc[0][qt][e], c_scale, sd[0]),
-                                     __builtin_fmaf(s_acc[0][qt][e + 1], c_scale, sd[1])));
-            }
-        } else {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[0][qt][e]);
-        }
-        mx = max_across_halves(mx);
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[0][qt][e]);
+        mx = max_across_halves(mx) * (EXACT ? c_scale : 1.f);       // c > 0: the maximum commutes with the scale
         row_max[qt] = (mx == -INFINITY || mx != mx) ? 0.f : mx;
         wave_max = fmaxf(wave_max, row_max[qt]);
     }
@@ -558,16 +537,16 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
 #pragma unroll
     for (int w = 1; w < NW; ++w) m_base = fmaxf(m_base, lds_ref[w]);
     if (wave_u == 0) {                 // tiles 0 and 1 were converted against a base of 0
-        lds_b[0][lane] -= m_base;
-        lds_b[1][lane] -= m_base;
+        lds_b[0][lane] -= m_base * unit;
+        lds_b[1][lane] -= m_base * unit;
     }
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
         const float gap = row_max[qt] - m_base;
         delta[qt] = gap < -Range<DT>::kMaxGap ? floorf(gap) : 0.f;
         m_run[qt] = m_base + delta[qt];
-        // the same scores, now relative to the reference (EXACT: m_base reaches them through the seeds in LDS)
-        const float back = EXACT ? delta[qt] * inv_c : m_run[qt];
+        // the same scores, now relative to the reference
+        const float back = m_run[qt] * unit;
 #pragma unroll
         for (int e = 0; e < 16; ++e) s_acc[0][qt][e] -= back;
     }
@@ -594,11 +573,11 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
             float sum[2];
             peek_bias(kb2);
             // slot a: keys 0..31 of tile j become probabilities; scores of keys 32..63; P V of keys 32..63 of tile j-1
-            slot(0, 1, kb, 0, kb, 1, kb3, 1, sum);
+            slot(0, 1, kb, 1, kb3, 1, sum);
             finish_slot(1, sum);
             commit_bias(j + 2, kb2);   // raw bias landed before the last barrier; published by the next one
             // slot b: keys 32..63 of tile j become probabilities; scores of keys 0..31 of tile j+1; P V of keys 0..31 of tile j
-            slot(1, 0, kb, 1, kb1, 0, kb, 0, sum);
+            slot(1, 0, kb1, 0, kb, 0, sum);
             finish_slot(0, sum);
 
             staged_wait(true);         // loads issued one iteration ago have landed
@@ -650,11 +629,9 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
                     float ex[16];
                     float mx = -INFINITY;
 #pragma unroll
-                    for (int e = 0; e < 16; e += 2) {
-                        const f32x2 sd = seed_pair(0, half, e);
-                        ex[e] = EXACT ? __builtin_fmaf(s_acc[0][qt][e], c_scale, sd[0]) : s_acc[0][qt][e];
-                        ex[e + 1] = EXACT ? __builtin_fmaf(s_acc[0][qt][e + 1], c_scale, sd[1]) : s_acc[0][qt][e + 1];
-                        mx = fmaxf(mx, fmaxf(ex[e], ex[e + 1]));
+                    for (int e = 0; e < 16; ++e) {
+                        ex[e] = EXACT ? s_acc[0][qt][e] * c_scale : s_acc[0][qt][e];
+                        mx = fmaxf(mx, ex[e]);
                     }
                     mx = fmaxf(max_across_halves(mx), m_row[qt]);
                     const float ref = mx == -INFINITY ? 0.f : mx;          // a row that has seen masked keys only
@@ -852,11 +829,6 @@ extern "C" int64_t come_attn_work_bytes(int64_t n_seq, int64_t total, int64_t n_
     return make_plan(n_seq, total, n_heads, max_seqlen, true).work_bytes;
 }
 
-// Process-wide: apply softmax_scale in fp32 behind the score MFMA instead of folding it into a 16-bit Q.
-static std::atomic<int> g_exact_scale{0};
-
-extern "C" int come_attn_set_exact_scale(int on) { return g_exact_scale.exchange(on != 0 ? 1 : 0); }
-
 // Address of this device's copy of `scratch` (nullptr + error message on failure).  The array's name is only a
 // host-side handle: the device address is asked for once per device, with that device current, and kept.
 static void *static_work_pointer() {
@@ -890,8 +862,10 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
                                 int64_t n_seq, int64_t total, int64_t n_heads, int64_t head_dim,
                                 const void *perkey_bias, int64_t max_seqlen, float softmax_scale, void *out,
                                 int64_t o_row_stride, int64_t o_head_stride, float *lse, void *work,
-                                int64_t work_bytes, bool static_work, void *stream) {
+                                int64_t work_bytes, bool static_work, int flags, void *stream) {
     clear_error();
+    COME_REQUIRE((flags & ~COME_ATTN_FOLD_SCALE) == 0, COME_ERR_INVALID,
+                 "come_attn_varlen_fwd: unknown bits in flags (%d)", flags);
     COME_REQUIRE(dtype == COME_BF16 || dtype == COME_F16, COME_ERR_UNSUPPORTED,
                  "come_attn_varlen_fwd: only fp16 and bf16 are supported");
     COME_REQUIRE(head_dim == 32 || head_dim == kHeadDim || head_dim == 128, COME_ERR_UNSUPPORTED,
@@ -984,7 +958,7 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
                  "come_attn_varlen_fwd: grid too large");
     const dim3 grid(static_cast<unsigned>(n_wg)), block(wide ? 512 : 256);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool exact = g_exact_scale.load(std::memory_order_relaxed) != 0;
+    const bool exact = (flags & COME_ATTN_FOLD_SCALE) == 0;
 #define COME_ATTN_LAUNCH(DT_, NW_)                                                                              \
     do {                                                                                                        \
         if (exact) hipLaunchKernelGGL((attn_fwd_pipe_kernel<DT_, NW_, true>), grid, block, 0, s, a);            \
@@ -1015,11 +989,11 @@ extern "C" int come_attn_varlen_fwd_ws(const void *q, const void *k, const void 
                                        int64_t n_seq, int64_t total, int64_t n_heads, int64_t head_dim,
                                        const void *perkey_bias, int64_t max_seqlen, float softmax_scale, void *out,
                                        int64_t o_row_stride, int64_t o_head_stride, float *lse, void *work,
-                                       int64_t work_bytes, void *stream) {
+                                       int64_t work_bytes, int flags, void *stream) {
     return attn_varlen_fwd_impl(q, k, v, dtype, q_row_stride, q_head_stride, k_row_stride, k_head_stride,
                                 v_row_stride, v_head_stride, cu_seqlens, n_seq, total, n_heads, head_dim,
                                 perkey_bias, max_seqlen, softmax_scale, out, o_row_stride, o_head_stride, lse,
-                                work, work_bytes, false, stream);
+                                work, work_bytes, false, flags, stream);
 }
 
 extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v, int dtype, int64_t q_row_stride,
@@ -1027,14 +1001,21 @@ extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v,
                                     int64_t v_row_stride, int64_t v_head_stride, const int32_t *cu_seqlens,
                                     int64_t n_seq, int64_t total, int64_t n_heads, int64_t head_dim,
                                     const void *perkey_bias, int64_t max_seqlen, float softmax_scale, void *out,
-                                    int64_t o_row_stride, int64_t o_head_stride, float *lse, void *stream) {
+                                    int64_t o_row_stride, int64_t o_head_stride, float *lse, int flags,
+                                    void *stream) {
     return attn_varlen_fwd_impl(q, k, v, dtype, q_row_stride, q_head_stride, k_row_stride, k_head_stride,
                                 v_row_stride, v_head_stride, cu_seqlens, n_seq, total, n_heads, head_dim,
                                 perkey_bias, max_seqlen, softmax_scale, out, o_row_stride, o_head_stride, lse,
-                                nullptr, 0, false, stream);
+                                nullptr, 0, false, flags, stream);
 }
 
-extern "C" int64_t come_attn_static_work_bytes(void) { return kStaticWorkBytes; }
+// Also takes the address of the current device's copy of the array, so that a caller who asks for the size before
+// its first launch (as a capturing caller has to, outside the capture) leaves nothing but kernel launches to the
+// entry point itself.  Returns -1 when that fails (come_last_error() says why).
+extern "C" int64_t come_attn_static_work_bytes(void) {
+    clear_error();
+    return static_work_pointer() != nullptr ? kStaticWorkBytes : -1;
+}
 
 extern "C" int come_attn_varlen_fwd_static(const void *q, const void *k, const void *v, int dtype,
                                            int64_t q_row_stride, int64_t q_head_stride, int64_t k_row_stride,
@@ -1042,9 +1023,9 @@ extern "C" int come_attn_varlen_fwd_static(const void *q, const void *k, const v
                                            const int32_t *cu_seqlens, int64_t n_seq, int64_t total, int64_t n_heads,
                                            int64_t head_dim, const void *perkey_bias, int64_t max_seqlen,
                                            float softmax_scale, void *out, int64_t o_row_stride,
-                                           int64_t o_head_stride, float *lse, void *stream) {
+                                           int64_t o_head_stride, float *lse, int flags, void *stream) {
     return attn_varlen_fwd_impl(q, k, v, dtype, q_row_stride, q_head_stride, k_row_stride, k_head_stride,
                                 v_row_stride, v_head_stride, cu_seqlens, n_seq, total, n_heads, head_dim,
                                 perkey_bias, max_seqlen, softmax_scale, out, o_row_stride, o_head_stride, lse,
-                                nullptr, 0, true, stream);
+                                nullptr, 0, true, flags, stream);
 }

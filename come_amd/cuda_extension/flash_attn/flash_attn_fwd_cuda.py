@@ -45,22 +45,16 @@ class _on_device:
         return False
 
 
-_PLACEHOLDERS: dict = {}
-
-
 def _placeholders(dev: torch.device, dtype: torch.dtype):
-    """The two results the forward never fills (attention probabilities, dropout RNG state): one empty tensor
-    and one two-element int64 tensor per device and dtype, never written by anything in this package."""
-    key = (dev, dtype)
-    if key not in _PLACEHOLDERS:
-        _PLACEHOLDERS[key] = (torch.empty((0,), dtype=dtype, device=dev),
-                              torch.zeros((2,), dtype=torch.int64, device=dev))
-    return _PLACEHOLDERS[key]
+    """The two results the forward never fills (attention probabilities, dropout RNG state): a fresh empty tensor
+    and a fresh two-element int64 tensor per call, as the reference returns (``flash_api.cpp:470-476, 489-493``), so
+    that no two callers ever hold the same object.  Neither costs a kernel launch."""
+    return torch.empty((0,), dtype=dtype, device=dev), torch.empty((2,), dtype=torch.int64, device=dev)
 
 
 def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
                      perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal,
-                     window_size_left, window_size_right, softcap, return_softmax, gen):
+                     window_size_left, window_size_right, softcap, return_softmax, gen, fold_scale=False):
     _check(q.dtype in (torch.float16, torch.bfloat16), "FlashAttention only support fp16 and bf16 data type")
     _check(k.dtype == q.dtype, "query and key must have the same dtype")
     _check(v.dtype == q.dtype, "query and value must have the same dtype")
@@ -129,7 +123,7 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
         padded = _varlen_fwd_impl(*(torch.nn.functional.pad(t, [0, kernel_width - head_size]) for t in (q, k, v)),
                                   None, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
                                   perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, False, is_causal,
-                                  window_size_left, window_size_right, softcap, return_softmax, gen)
+                                  window_size_left, window_size_right, softcap, return_softmax, gen, fold_scale)
         narrow = padded[0][..., :head_size]
         if out_ is not None:
             _check(out_.dtype == q.dtype and tuple(out_.shape) == (total_q, num_heads, head_size),
@@ -168,7 +162,8 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
                 cu_seqlens_q.data_ptr(), batch_size, total_q, num_heads, head_size,
                 _lib.ptr(perkey_bias), max_seqlen_k, float(softmax_scale),
                 out.data_ptr(), out.stride(0), out.stride(1), softmax_lse.data_ptr(),
-                _lib.ptr(work), work_bytes, _lib.current_stream(dev)))
+                _lib.ptr(work), work_bytes, _lib.COME_ATTN_FOLD_SCALE if fold_scale else 0,
+                _lib.current_stream(dev)))
         else:
             out.zero_()
             softmax_lse.fill_(math.inf)
@@ -177,20 +172,24 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
 
 def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
                max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal,
-               window_size_left, window_size_right, softcap, return_softmax, gen=None):
-    """Forward pass (variable length).  Returns ``[out, softmax_lse, p, rng_state]``."""
+               window_size_left, window_size_right, softcap, return_softmax, gen=None, *, fold_scale=False):
+    """Forward pass (variable length).  Returns ``[out, softmax_lse, p, rng_state]``.
+
+    ``fold_scale`` (keyword only, not in the reference): fold ``softmax_scale`` into a 16-bit q instead of applying
+    it in fp32 to every score (``COME_ATTN_FOLD_SCALE`` of the C ABI); for callers that know their logits stay within
+    about +-10 nats."""
     return _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table,
                             alibi_slopes, None, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                             zero_tensors, is_causal, window_size_left, window_size_right, softcap,
-                            return_softmax, gen)
+                            return_softmax, gen, fold_scale)
 
 
 def varlen_fwd_w_perkey_bias(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table,
                              alibi_slopes, perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                              zero_tensors, is_causal, window_size_left, window_size_right, softcap,
-                             return_softmax, gen=None):
-    """Forward pass (variable length) with a per-key additive bias."""
+                             return_softmax, gen=None, *, fold_scale=False):
+    """Forward pass (variable length) with a per-key additive bias (``fold_scale``: see :func:`varlen_fwd`)."""
     return _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table,
                             alibi_slopes, perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                             zero_tensors, is_causal, window_size_left, window_size_right, softcap,
-                            return_softmax, gen)
+                            return_softmax, gen, fold_scale)

@@ -37,6 +37,21 @@ typedef enum come_dtype {
     COME_BF16 = 2
 } come_dtype;
 
+/*
+ * Bits of the `flags` argument of come_attn_varlen_fwd / _ws / _static (head_dim 64; the other widths always use
+ * the arithmetic of flags = 0).  They are per call: nothing in the library remembers them.
+ *
+ *   0                      softmax_scale is applied in fp32 to every score, q enters the matrix unit as it is and
+ *                          bias / scale is added to the raw scores: the reference's arithmetic
+ *                          (src/cuda_extension/flash_attn/src/flash_fwd_kernel.h:30-55, src/softmax.h:76-88).
+ *   COME_ATTN_FOLD_SCALE   q is multiplied by softmax_scale * log2(e) once and rounded back to `dtype`, which saves
+ *                          one vector instruction per score (about 10 % of the run time) and moves a logit by up to
+ *                          2^-9 of its size: inside 1e-2 max-abs / 1e-3 mean-abs for logits within about +-10 nats
+ *                          (q / k LayerNorm with gains near 1), outside it from about +-20 nats on.  A caller that
+ *                          knows such a bound for its logits may set it; nothing else should.
+ */
+enum { COME_ATTN_FOLD_SCALE = 1 };
+
 /* Library version (major * 10000 + minor * 100 + patch). */
 int come_version(void);
 
@@ -193,8 +208,8 @@ int come_select_plan(const void *conf, int dtype, int64_t batch, int64_t frames,
  *   perkey_bias [total] of `dtype`, or NULL for plain attention
  *   max_seqlen  upper bound of the segment lengths (sizes the launch grid)
  *   out       [total, n_heads, head_dim] of `dtype`, strides in elements
- *   lse       [n_heads, total] float: logsumexp of the biased, scaled scores (within 1e-2: the
- *             scaled q is rounded to 16 bits); may be NULL
+ *   lse       [n_heads, total] float: logsumexp of the biased, scaled scores; may be NULL
+ *   flags     0 or COME_ATTN_FOLD_SCALE (above)
  * head_dim is 32, 64 or 128 (the reference instantiates 32 ... 256 in steps of 32,
  * src/cuda_extension/flash_attn/src/flash_fwd_launch_template.h:174-330; callers pad other widths up to 128 with
  * zero columns, which changes neither q . k nor the other output columns).
@@ -203,7 +218,7 @@ int come_select_plan(const void *conf, int dtype, int64_t batch, int64_t frames,
  * that type can hold within one 32-key step (2^127 for COME_BF16, about 2^15 for COME_F16) computes its query block
  * again with a running maximum, so the result is right for any finite scores.
  * head_dim 32 and 128: one 32-query tile per wavefront, scale and bias applied to the fp32 scores (as with
- * come_attn_set_exact_scale(1)), running maximum per row; no work buffer is used.
+ * flags = 0), running maximum per row; no work buffer is used.
  *
  * Stands in for varlen_fwd / varlen_fwd_w_perkey_bias
  * (src/cuda_extension/flash_attn/flash_api.cpp:291-607; kernel
@@ -219,18 +234,7 @@ int come_attn_varlen_fwd(const void *q, const void *k, const void *v, int dtype,
                          int64_t n_heads, int64_t head_dim,
                          const void *perkey_bias, int64_t max_seqlen, float softmax_scale,
                          void *out, int64_t o_row_stride, int64_t o_head_stride,
-                         float *lse, void *stream);
-
-/*
- * come_attn_set_exact_scale — process-wide switch for how softmax_scale reaches the scores; returns the previous
- * setting.
- *   0 (default)  Q is multiplied by softmax_scale * log2(e) once and rounded back to `dtype`: a logit moves by up to
- *                2^-9 of its size, which is inside the stated tolerance (1e-2 max-abs) for logits up to some ten nats;
- *   1            Q enters the MFMA as it is and the scale is applied in fp32 to every score, as the reference applies
- *                it (src/cuda_extension/flash_attn/src/softmax.h:76-88): one more vector instruction per score,
- *                about 10 % slower, for callers whose logits reach tens of nats (large q / k norm gains).
- */
-int come_attn_set_exact_scale(int on);
+                         float *lse, int flags, void *stream);
 
 /*
  * come_attn_varlen_fwd_ws — the same operator with a caller-supplied work buffer.  When the launch would end
@@ -240,7 +244,9 @@ int come_attn_set_exact_scale(int on);
  *
  *   work, work_bytes   device buffer, 16-byte aligned, of at least come_attn_work_bytes(...) bytes; NULL or a
  *                      smaller buffer makes the call identical to come_attn_varlen_fwd
- * come_attn_work_bytes returns 0 when a launch of that shape would not use a buffer.
+ * come_attn_work_bytes returns 0 when a launch of that shape would not use a buffer.  The buffer is used for
+ * head_dim 64 only: the size query does not know the head width, so callers of the 32- and 128-wide instances pass
+ * NULL / 0 instead of allocating what it returns.
  *
  * No counterpart in the reference (its kernel has a split-KV variant for decoding only,
  * src/cuda_extension/flash_attn/src/flash_fwd_launch_template.h:99-157, unreachable from the varlen forward).
@@ -254,7 +260,7 @@ int come_attn_varlen_fwd_ws(const void *q, const void *k, const void *v, int dty
                             int64_t n_heads, int64_t head_dim,
                             const void *perkey_bias, int64_t max_seqlen, float softmax_scale,
                             void *out, int64_t o_row_stride, int64_t o_head_stride,
-                            float *lse, void *work, int64_t work_bytes, void *stream);
+                            float *lse, void *work, int64_t work_bytes, int flags, void *stream);
 
 /*
  * come_attn_varlen_fwd_static — come_attn_varlen_fwd_ws without a buffer argument and without any allocation:
@@ -268,6 +274,10 @@ int come_attn_varlen_fwd_ws(const void *q, const void *k, const void *v, int dty
  * stream are ordered by the stream.  Nothing in the array has to be cleared between calls: every piece is
  * written in full before the combining kernel of the same call reads it.
  *
+ * come_attn_static_work_bytes() also looks up the address of the current device's copy of the array (-1 if that
+ * fails); a caller that records launches into a graph calls it once per device before the capture, so that the
+ * entry point itself makes nothing but kernel launches.
+ *
  * No counterpart in the reference.  It is for callers that cannot allocate device memory around the call: code
  * under HIP graph capture, tight serving loops, harnesses that forbid allocation.
  */
@@ -280,7 +290,7 @@ int come_attn_varlen_fwd_static(const void *q, const void *k, const void *v, int
                                 int64_t n_heads, int64_t head_dim,
                                 const void *perkey_bias, int64_t max_seqlen, float softmax_scale,
                                 void *out, int64_t o_row_stride, int64_t o_head_stride,
-                                float *lse, void *stream);
+                                float *lse, int flags, void *stream);
 
 /*
  * come_qk_norm_rope — attention prologue, in place on the packed projection output:

@@ -43,7 +43,7 @@ def test_version_and_error_string():
                                 None, None, None, None, None) == 2
     assert b"dtype" in lib.come_last_error()
     assert lib.come_attn_varlen_fwd(None, None, None, _lib.COME_BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 96,
-                                    None, 10, 0.125, None, 64, 64, None, None) == 2
+                                    None, 10, 0.125, None, 64, 64, None, 0, None) == 2
     assert b"head_dim" in lib.come_last_error()
     assert lib.come_select_work_bytes(1, 16, 37, 37, 3, 3) >= 16 * 144 * 4
 
@@ -102,15 +102,17 @@ def test_every_entry_point_rejects_bad_arguments_on_the_host():
     rejected(lib.come_select_windows(None, F32, 1, 1, 6, 6, 3, 3, 7, 0.5, None, None, None, 0, None), "mode")
     rejected(lib.come_select_windows(None, F32, 1, 1, 6, 6, 3, 3, 0, 1.5, None, None, None, 0, None), "threshold")
     rejected(lib.come_attn_varlen_fwd(None, None, None, F32, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 64,
-                                      None, 10, 0.125, None, 64, 64, None, None), "fp16 and bf16")
+                                      None, 10, 0.125, None, 64, 64, None, 0, None), "fp16 and bf16")
     rejected(lib.come_attn_varlen_fwd(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 0, 10, 1, 64,
-                                      None, 10, 0.125, None, 64, 64, None, None), "batch size")
+                                      None, 10, 0.125, None, 64, 64, None, 0, None), "batch size")
     rejected(lib.come_attn_varlen_fwd(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 64,
-                                      None, 10, -1.0, None, 64, 64, None, None), "softmax_scale")
+                                      None, 10, -1.0, None, 64, 64, None, 0, None), "softmax_scale")
     rejected(lib.come_attn_varlen_fwd(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 64,
-                                      None, 10, 0.125, None, 64, 64, None, None), "NULL")
+                                      None, 10, 0.125, None, 64, 64, None, 0, None), "NULL")
+    rejected(lib.come_attn_varlen_fwd(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 64,
+                                      None, 10, 0.125, None, 64, 64, None, 6, None), "flags")
     rejected(lib.come_attn_varlen_fwd_ws(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 48,
-                                         None, 10, 0.125, None, 64, 64, None, None, 0, None), "head_dim")
+                                         None, 10, 0.125, None, 64, 64, None, None, 0, 0, None), "head_dim")
     rejected(lib.come_qk_norm_rope(None, None, F32, 64, 64, 64, 64, 4, 1, 64, 1, None, None, None, None, 1e-5,
                                    None, None, None, 0, None), "bf16 or fp16")
     rejected(lib.come_qk_norm_rope(None, None, BF16, 64, 64, 64, 64, 4, 1, 32, 1, None, None, None, None, 1e-5,

@@ -18,7 +18,7 @@ from come_amd.cuda_extension import (
     flash_attn_varlen_qkvpacked_func_w_perkey_bias,
     infer_flash_attn_varlen_max_seqlen,
 )
-from come_amd.cuda_extension.flash_attn import flash_attn_fwd_cuda, set_exact_softmax_scale
+from come_amd.cuda_extension.flash_attn import flash_attn_fwd_cuda
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -28,13 +28,10 @@ SEGMENT_SETS = [[32, 48, 24, 24], [56, 49, 23], [128], [60, 40], [50], [128, 256
                 [1], [3, 1, 2], [65], [257, 31], [700, 333, 64], [1000]]
 
 
-@pytest.fixture
-def exact_scale():
-    """Runs a test with softmax_scale applied in fp32 to every score (the reference's arithmetic) and restores the
-    default (scale folded into a 16-bit Q) afterwards."""
-    before = set_exact_softmax_scale(True)
-    yield
-    set_exact_softmax_scale(before)
+# How softmax_scale reaches the scores is a per-call choice (``scale_mode``): "exact" - in fp32 on every score, the
+# reference's arithmetic and what a tensor without a known logit bound gets ("auto"); "folded" - multiplied into a
+# 16-bit q once, for logits within about +-10 nats.  Cases whose logits stay small run in both.
+MODES = ["exact", "folded"]
 
 
 def _cu(lens):
@@ -49,7 +46,7 @@ def _compare(out, ref):
     torch.testing.assert_close(out, ref, atol=1e-2, rtol=1e-2)
 
 
-def _run(lens, H, dtype, bias_kind="weights", scale=None, return_lse=False):
+def _run(lens, H, dtype, bias_kind="weights", scale=None, return_lse=False, mode="auto"):
     P, D = sum(lens), 64
     qkv = torch.randn(P, 3, H, D).to(dtype)
     if bias_kind == "weights":
@@ -62,39 +59,68 @@ def _run(lens, H, dtype, bias_kind="weights", scale=None, return_lse=False):
     ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias, softmax_scale=scale)
     args = (qkv.to(DEV), cu.to(DEV), max(lens))
     if bias is None:
-        res = flash_attn_varlen_qkvpacked_func(*args, softmax_scale=scale, return_attn_probs=return_lse)
+        res = flash_attn_varlen_qkvpacked_func(*args, softmax_scale=scale, return_attn_probs=return_lse,
+                                               scale_mode=mode)
     else:
         res = flash_attn_varlen_qkvpacked_func_w_perkey_bias(*args, perkey_bias=bias.to(DEV), softmax_scale=scale,
-                                                             return_attn_probs=return_lse)
+                                                             return_attn_probs=return_lse, scale_mode=mode)
     if return_lse:
         out, lse, _ = res
-        torch.testing.assert_close(lse.cpu(), ref_lse, atol=2e-3, rtol=1e-3)
+        # folded: the scaled q is rounded to 16 bits, a logit (and with it lse) moves by up to 2^-9 of its size
+        torch.testing.assert_close(lse.cpu(), ref_lse, atol=1e-2 if mode == "folded" else 2e-3, rtol=1e-3)
     else:
         out = res
     assert out.shape == (P, H, D) and out.dtype == dtype
     _compare(out, ref)
 
 
+@pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("lens", SEGMENT_SETS, ids=[str(s) for s in SEGMENT_SETS])
-def test_bias_matches_closed_form_bf16(lens):
-    _run(lens, H=4, dtype=torch.bfloat16)
+def test_bias_matches_closed_form_bf16(lens, mode):
+    _run(lens, H=4, dtype=torch.bfloat16, mode=mode, return_lse=True)
 
 
+@pytest.mark.parametrize("mode", ["auto"] + MODES)
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
-def test_dtypes(dtype):
-    _run([64, 64], H=4, dtype=dtype)
-    _run([100, 150, 50], H=2, dtype=dtype, bias_kind="counts")
+def test_dtypes(dtype, mode):
+    _run([64, 64], H=4, dtype=dtype, mode=mode)
+    _run([100, 150, 50], H=2, dtype=dtype, bias_kind="counts", mode=mode)
 
 
+@pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("lens", [[128, 256], [300, 77], [2048, 1111]])
-def test_plain_attention_and_lse(lens):
-    _run(lens, H=2, dtype=torch.bfloat16, bias_kind=None, return_lse=True)
-    _run(lens, H=2, dtype=torch.bfloat16, bias_kind="counts", return_lse=True)
+def test_plain_attention_and_lse(lens, mode):
+    _run(lens, H=2, dtype=torch.bfloat16, bias_kind=None, return_lse=True, mode=mode)
+    _run(lens, H=2, dtype=torch.bfloat16, bias_kind="counts", return_lse=True, mode=mode)
 
 
-def test_sixteen_heads_long_segments_and_other_scale():
-    _run([3000, 1500], H=16, dtype=torch.bfloat16, bias_kind="counts")
-    _run([500, 260], H=3, dtype=torch.bfloat16, scale=0.2)           # scale that is not a power of two
+@pytest.mark.parametrize("mode", MODES)
+def test_sixteen_heads_long_segments_and_other_scale(mode):
+    _run([3000, 1500], H=16, dtype=torch.bfloat16, bias_kind="counts", mode=mode)
+    _run([500, 260], H=3, dtype=torch.bfloat16, scale=0.2, mode=mode)           # scale that is not a power of two
+
+
+def test_scale_mode_is_validated_and_auto_follows_the_bound_on_the_tensor():
+    """"auto" folds the scale only for a tensor that carries a small enough ``come_qk_bound`` (set by
+    ``prepare_packed_self_attention_qkv``); results are bit-identical to the explicitly named mode."""
+    lens, H = [700, 333], 4
+    P = sum(lens)
+    g = torch.Generator().manual_seed(3)
+    qkv = torch.randn(P, 3, H, 64, generator=g).bfloat16().to(DEV)
+    bias = torch.where(torch.rand(P, generator=g) < 0.3, math.log(9.0), 0.0).bfloat16().to(DEV)
+    cu = _cu(lens).to(DEV)
+    run = lambda t, **kw: flash_attn_varlen_qkvpacked_func_w_perkey_bias(t, cu, max(lens), perkey_bias=bias, **kw)
+    exact, folded = run(qkv, scale_mode="exact"), run(qkv, scale_mode="folded")
+    assert not torch.equal(exact, folded)
+    assert torch.equal(run(qkv), exact)                         # no bound known: the reference's arithmetic
+    tagged = qkv.clone()
+    tagged.come_qk_bound = 64.0                                 # 64 * 0.125 = 8 nats
+    assert torch.equal(run(tagged), folded)
+    tagged.come_qk_bound = 256.0                                # 32 nats
+    assert torch.equal(run(tagged), exact)
+    assert torch.equal(run(tagged, scale_mode="folded"), folded)
+    with pytest.raises(ValueError, match="scale_mode"):
+        run(qkv, scale_mode="fast")
 
 
 def test_zero_bias_equals_plain_operator():
@@ -131,9 +157,9 @@ def test_count_bias_equals_key_duplication():
     assert float(diff.max()) <= 2e-2 and float(diff.mean()) <= 2e-3
 
 
-def test_sharp_logits_with_exact_scale(exact_scale):
-    """The case that needs 8e-2 with the scale folded into a 16-bit Q (late_rows below: logits of up to +-35 nats
-    with near-ties between the leading keys) meets the ordinary tolerance when the scale is applied in fp32."""
+def test_sharp_logits_in_the_default_mode():
+    """Logits of up to +-35 nats with near-ties between the leading keys (late_rows below) meet the ordinary tolerance
+    in the default mode, where the scale is applied in fp32; folded into a 16-bit q the case needs 8e-2."""
     L, H = 1500, 2
     qkv = torch.randn(L, 3, H, 64).bfloat16()
     qkv[:, 1, :, :] *= torch.linspace(0.2, 6.0, L)[:, None, None].bfloat16()
@@ -150,21 +176,22 @@ def test_sharp_logits_with_exact_scale(exact_scale):
 
 @pytest.mark.parametrize("gain", [1, 2, 4])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
-def test_layernormed_qk_with_gains_exact_scale(gain, dtype, exact_scale):
+def test_layernormed_qk_with_gains(gain, dtype):
     """What the real caller feeds the operator (reference vggt/module/bias_attention.py:100-137: q and k are
-    LayerNorm'd per head, so |q| = |k| = 8 * gain and logits reach 8 * gain^2 nats), at the ordinary tolerance."""
+    LayerNorm'd per head, so |q| = |k| = 8 * gain and logits reach 8 * gain^2 nats), at the ordinary tolerance, through
+    the default call."""
     _check_layernormed(gain, dtype)
 
 
-def test_layernormed_qk_unit_gain_default_mode():
-    """With unit gains (logits within +-8 nats) the default mode - scale folded into a 16-bit Q - is inside the
-    tolerance as well; from a gain of 2 on it is not (measured max-abs 2.3e-2 at gain 2, 1.2e-1 at gain 4 in bf16),
-    which is what the exact mode is for."""
-    _check_layernormed(1, torch.bfloat16)
-    _check_layernormed(1, torch.float16)
+def test_layernormed_qk_unit_gain_folded_mode():
+    """With unit gains (logits within +-8 nats) folding the scale into a 16-bit q is inside the tolerance as well;
+    from a gain of 2 on it is not (measured max-abs 2.3e-2 at gain 2, 1.2e-1 at gain 4 in bf16), which is why only
+    tensors with a known small bound get it."""
+    _check_layernormed(1, torch.bfloat16, mode="folded")
+    _check_layernormed(1, torch.float16, mode="folded")
 
 
-def _check_layernormed(gain, dtype):
+def _check_layernormed(gain, dtype, mode="auto"):
     lens, H = [700, 333, 64], 4
     P = sum(lens)
     g = torch.Generator().manual_seed(gain)
@@ -176,14 +203,15 @@ def _check_layernormed(gain, dtype):
     cu = _cu(lens)
     ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias)
     out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), max(lens),
-                                                                 perkey_bias=bias.to(DEV), return_attn_probs=True)
+                                                                 perkey_bias=bias.to(DEV), return_attn_probs=True,
+                                                                 scale_mode=mode)
     diff = (out.float().cpu() - ref).abs()
     torch.testing.assert_close(out.float().cpu(), ref, atol=1e-2, rtol=1e-2)
     assert float(diff.mean()) <= MEAN_ABS
     torch.testing.assert_close(lse.cpu(), ref_lse, atol=5e-3, rtol=1e-3)
 
 
-@pytest.mark.parametrize("mode", ["default", "exact"])
+@pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("dtype,jump", [(torch.bfloat16, 100.0), (torch.bfloat16, 300.0), (torch.float16, 12.0),
                                         (torch.float16, 30.0)], ids=["bf16+100", "bf16+300", "f16+12", "f16+30"])
 def test_late_key_beyond_the_range_of_the_stored_probabilities(dtype, jump, mode):
@@ -192,32 +220,54 @@ def test_late_key_beyond_the_range_of_the_stored_probabilities(dtype, jump, mode
     value saturates from about 11 nats on).  The workgroup notices and computes its block again with a running
     maximum, so the result meets the ordinary tolerance.  Several such keys, in the first tile, at tile borders and
     in a second, short segment (tail block)."""
-    before = set_exact_softmax_scale(mode == "exact")
-    try:
-        lens, H = [1500, 90], 2
-        P = sum(lens)
-        g = torch.Generator().manual_seed(int(jump))
-        qkv = torch.randn(P, 3, H, 64, generator=g).to(dtype)
-        bias = torch.zeros(P)
-        bias[700] = jump                       # one step
-        bias[1023] = 2 * jump                  # a second one on top, last key of a tile
-        bias[1024] = 2 * jump - 1.0            # and a near-tie right behind it, first key of the next tile
-        bias[1500 + 40] = jump                 # second segment: inside its only query block
-        bias = bias.to(dtype)
-        assert bool(torch.isfinite(bias.float()).all())
-        cu = _cu(lens)
-        ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias)
-        out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), max(lens),
-                                                                     perkey_bias=bias.to(DEV), return_attn_probs=True)
-        assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(lse).all())
-        # two near-tied keys carry every row: the result is a 0.73 / 0.27 mix of two value rows, and rounding those
-        # two probabilities and the result to 16 bits alone costs about 2^-9 of the value (as in the reference's kernel)
-        diff = (out.float().cpu() - ref).abs()
-        torch.testing.assert_close(out.float().cpu(), ref, atol=1e-2, rtol=1e-2)     # the reference's own criterion
-        assert float(diff.mean()) <= MEAN_ABS + 2.0 ** -9 * float(ref.abs().mean()), f"mean-abs {float(diff.mean())}"
-        torch.testing.assert_close(lse.cpu(), ref_lse, atol=2e-2 if mode == "default" else 5e-3, rtol=1e-3)
-    finally:
-        set_exact_softmax_scale(before)
+    lens, H = [1500, 90], 2
+    P = sum(lens)
+    g = torch.Generator().manual_seed(int(jump))
+    qkv = torch.randn(P, 3, H, 64, generator=g).to(dtype)
+    bias = torch.zeros(P)
+    bias[700] = jump                       # one step
+    bias[1023] = 2 * jump                  # a second one on top, last key of a tile
+    bias[1024] = 2 * jump - 1.0            # and a near-tie right behind it, first key of the next tile
+    bias[1500 + 40] = jump                 # second segment: inside its only query block
+    bias = bias.to(dtype)
+    assert bool(torch.isfinite(bias.float()).all())
+    cu = _cu(lens)
+    ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias)
+    out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), max(lens),
+                                                                 perkey_bias=bias.to(DEV), return_attn_probs=True,
+                                                                 scale_mode=mode)
+    assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(lse).all())
+    # two near-tied keys carry every row: the result is a 0.73 / 0.27 mix of two value rows, and rounding those
+    # two probabilities and the result to 16 bits alone costs about 2^-9 of the value (as in the reference's kernel)
+    diff = (out.float().cpu() - ref).abs()
+    torch.testing.assert_close(out.float().cpu(), ref, atol=1e-2, rtol=1e-2)     # the reference's own criterion
+    assert float(diff.mean()) <= MEAN_ABS + 2.0 ** -9 * float(ref.abs().mean()), f"mean-abs {float(diff.mean())}"
+    torch.testing.assert_close(lse.cpu(), ref_lse, atol=2e-2 if mode == "folded" else 5e-3, rtol=1e-3)
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("jump", [80.0, 84.0, 87.0, 88.0])
+def test_late_key_just_inside_the_float_range_with_large_values(jump, mode):
+    """A late key that beats its row by 80 - 88 nats leaves a probability of 2^115 - 2^127 relative to the old reference
+    point: still finite, so the row sum alone would not give it away, but multiplied by values of size 8 and added up
+    over the keys of a step the fp32 outputs would overflow.  The redo threshold leaves that headroom."""
+    L, H = 900, 2
+    g = torch.Generator().manual_seed(int(jump))
+    qkv = torch.randn(L, 3, H, 64, generator=g)
+    qkv[:, 2] *= 8.0
+    qkv = qkv.bfloat16()
+    bias = torch.zeros(L)
+    bias[500] = jump
+    bias[501:520] = jump - 0.5             # a cluster right behind it: their products with v add up
+    bias = bias.bfloat16()
+    cu = _cu([L])
+    ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias)
+    out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), L, perkey_bias=bias.to(DEV),
+                                                                 return_attn_probs=True, scale_mode=mode)
+    assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(lse).all())
+    # outputs are 8 times the usual size and their rounding errors with them: the usual bounds on out / 8
+    torch.testing.assert_close(out.float().cpu() / 8, ref / 8, atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(lse.cpu(), ref_lse, atol=2e-2 if mode == "folded" else 5e-3, rtol=1e-3)
 
 
 def test_key_beyond_the_range_inside_a_key_split_piece():
@@ -267,16 +317,25 @@ def test_reference_point_moves(kind):
     out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), L, perkey_bias=bias.to(DEV),
                                                                  return_attn_probs=True)
     assert bool(torch.isfinite(out).all())
+    if kind != "late_rows":
+        _compare(out, ref)
+    else:
+        # sharp rows whose outputs reach 4: a bf16 output in [2, 4) is only known to 2^-7 = 7.8e-3, and two leading
+        # probabilities rounded to bf16 (as in the reference's kernel) add as much, so the absolute bound cannot hold
+        # there; the reference's own criterion (atol = rtol = 1e-2 per element) and the mean bound do
+        torch.testing.assert_close(out.float().cpu(), ref, atol=1e-2, rtol=1e-2)
+        assert float((out.float().cpu() - ref).abs().mean()) <= MEAN_ABS
+    torch.testing.assert_close(lse.cpu(), ref_lse, atol=5e-3, rtol=1e-3)
     if kind == "late_rows":
-        # logits of up to +-35 nats with near-ties between the leading keys: the kernel multiplies Q by
-        # softmax_scale * log2(e) once and rounds it back to 16 bit, an error in the logit that grows with its
-        # magnitude (about 1e-3 * |logit| / sqrt(head_dim) bits); at this extreme it shows as a few 1e-2
+        # logits of up to +-35 nats with near-ties between the leading keys: with softmax_scale * log2(e) folded into
+        # a 16-bit q the error in a logit grows with its magnitude (about 1e-3 * |logit| / sqrt(head_dim) bits) and
+        # shows as a few 1e-2 at this extreme - the case the default mode exists for
+        out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), L,
+                                                                     perkey_bias=bias.to(DEV), return_attn_probs=True,
+                                                                     scale_mode="folded")
         diff = (out.float().cpu() - ref).abs()
         assert float(diff.max()) <= 8e-2 and float(diff.mean()) <= 5e-3, (float(diff.max()), float(diff.mean()))
         torch.testing.assert_close(lse.cpu(), ref_lse, atol=5e-2, rtol=2e-3)
-        return
-    _compare(out, ref)
-    torch.testing.assert_close(lse.cpu(), ref_lse, atol=5e-3, rtol=1e-3)
 
 
 def test_fp16_reference_point_moves_within_its_narrow_range():
@@ -317,7 +376,7 @@ def test_rows_of_very_different_magnitude_in_one_workgroup():
     assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(lse).all())
     _compare(out, ref)
     torch.testing.assert_close(lse.cpu()[:, ~big], ref_lse[:, ~big], atol=5e-3, rtol=1e-3)
-    torch.testing.assert_close(lse.cpu()[:, big], ref_lse[:, big], atol=0.3, rtol=1e-3)   # 80 nats +- the 16-bit Q scaling
+    torch.testing.assert_close(lse.cpu()[:, big], ref_lse[:, big], atol=2e-2, rtol=1e-3)  # 80 nats
 
 
 def test_strided_views_and_separate_tensors():
@@ -441,9 +500,10 @@ def test_random_shapes_with_lengths_at_tile_borders(seed):
             pad[i][..., :64] = qkv[:, i].to(DEV)
         q, k, v = (t[..., :64] for t in pad)                                         # three row / head strides
     out_ = torch.full((P, H, 64), float("nan"), dtype=dtype, device=DEV) if pick([True, False]) else None
+    fold = seed % 2 == 1                   # alternate between the two ways of applying the scale
     out, lse, _, _ = flash_attn_fwd_cuda.varlen_fwd_w_perkey_bias(
         q, k, v, out_, cu.to(DEV), cu.to(DEV), None, None, None, None, None if bias is None else bias.to(DEV),
-        max_len, max_len, 0.0, scale, False, False, -1, -1, 0.0, False, None)
+        max_len, max_len, 0.0, scale, False, False, -1, -1, 0.0, False, None, fold_scale=fold)
     if out_ is not None:
         assert out.data_ptr() == out_.data_ptr()
     assert bool(torch.isfinite(out).all())
@@ -453,8 +513,9 @@ def test_random_shapes_with_lengths_at_tile_borders(seed):
     diff = (out.float().cpu() - ref).abs()
     torch.testing.assert_close(out.float().cpu(), ref, atol=1e-2, rtol=1e-2)
     assert float(diff.mean()) <= MEAN_ABS + 2.0 ** -9 * float(ref.abs().mean()), f"mean-abs {float(diff.mean())}"
-    # the kernel rounds the scaled Q to 16 bits: a logit, and with it lse, moves by up to 2^-9 of the logit's size
-    torch.testing.assert_close(lse.cpu(), ref_lse, atol=1e-2, rtol=1e-3)
+    # the row sum is taken from the probabilities as rounded to 16 bits (so that numerator and denominator of the
+    # output agree): for rows of one or two keys that is up to 2^-9 of the sum, 2e-3 in lse, on top of the rest
+    torch.testing.assert_close(lse.cpu(), ref_lse, atol=1e-2 if fold else 4e-3, rtol=1e-3)
 
 
 def test_bias_of_minus_infinity_masks_keys():

@@ -24,7 +24,7 @@ def single_pass(qkv, cu, max_len, bias):
     _lib.check(lib.come_attn_varlen_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.dtype_code(qkv.dtype),
                                         q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
                                         cu.data_ptr(), cu.numel() - 1, P, H, D, bias.data_ptr(), max_len, 0.125,
-                                        out.data_ptr(), out.stride(0), out.stride(1), lse.data_ptr(),
+                                        out.data_ptr(), out.stride(0), out.stride(1), lse.data_ptr(), 0,
                                         _lib.current_stream(qkv.device)))
     return out, lse
 
@@ -78,7 +78,7 @@ def test_work_buffer_rules():
     _lib.check(lib.come_attn_varlen_fwd_ws(q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.COME_BF16, q.stride(0), q.stride(1),
                                            k.stride(0), k.stride(1), v.stride(0), v.stride(1), cu.data_ptr(), 1, P, H, D,
                                            bias.data_ptr(), P, 0.125, out.data_ptr(), out.stride(0), out.stride(1), None,
-                                           small.data_ptr(), small.numel(), _lib.current_stream(qkv.device)))
+                                           small.data_ptr(), small.numel(), 0, _lib.current_stream(qkv.device)))
     assert torch.equal(out, ref_out)
 
 

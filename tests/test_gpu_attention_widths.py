@@ -181,11 +181,11 @@ def test_strided_views_and_the_three_entry_points(D):
                 dev_bias.data_ptr(), max(lens), D ** -0.5, out.data_ptr(), out.stride(0), out.stride(1), lse.data_ptr())
         stream = _lib.current_stream(torch.device(DEV))
         if entry == "plain":
-            rc = lib.come_attn_varlen_fwd(*head, stream)
+            rc = lib.come_attn_varlen_fwd(*head, 0, stream)
         elif entry == "ws":
-            rc = lib.come_attn_varlen_fwd_ws(*head, None, 0, stream)
+            rc = lib.come_attn_varlen_fwd_ws(*head, None, 0, 0, stream)
         else:
-            rc = lib.come_attn_varlen_fwd_static(*head, stream)
+            rc = lib.come_attn_varlen_fwd_static(*head, 0, stream)
         _lib.check(rc)
         torch.cuda.synchronize()
         _compare(out, ref)
@@ -203,7 +203,7 @@ def test_unsupported_width_is_rejected_by_the_library():
     rc = lib.come_attn_varlen_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.dtype_code(torch.bfloat16),
                                   q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
                                   cu.data_ptr(), 1, 8, 1, 96, None, 8, 0.1, out.data_ptr(), out.stride(0),
-                                  out.stride(1), None, _lib.current_stream(torch.device(DEV)))
+                                  out.stride(1), None, 0, _lib.current_stream(torch.device(DEV)))
     assert rc == 2                                           # COME_ERR_UNSUPPORTED
     assert b"head_dim" in lib.come_last_error()
 

@@ -77,3 +77,33 @@ def test_predictor_adapter_calls_reference_style_modules_with_the_shape():
     torch.testing.assert_close(plain.reshape(6, 20), want, atol=1e-2, rtol=1e-2)
     with pytest.raises(ValueError, match="one confidence per patch"):
         run_predictor(lambda t: t.float(), feature)
+
+
+def test_scale_mode_choice_follows_the_bound_attached_by_the_prologue():
+    """Host logic only: the norm bound of a LayerNorm'd head from its gain and bias, and the decision the attention
+    operators derive from a tensor's ``come_qk_bound`` (no bound: never folded)."""
+    from come_amd.common.qkv import _norm_bound
+    from come_amd.cuda_extension.flash_attn import FOLD_SCALE_MAX_LOGIT, _fold_scale
+
+    ln = torch.nn.LayerNorm(64)
+    assert _norm_bound(ln.weight, ln.bias, 64, torch.bfloat16) == pytest.approx(8.0)
+    with torch.no_grad():
+        ln.weight.fill_(0.5)
+        ln.weight[3] = -2.0
+        ln.bias.fill_(0.25)
+    assert _norm_bound(ln.weight, ln.bias, 64, torch.bfloat16) == pytest.approx(8.0 * 2.0 + 0.25 * 8.0)   # new version, new value
+    assert _norm_bound(None, None, 64, torch.float16) == pytest.approx(8.0)
+    # the bound really bounds the norm of any normalised head
+    x = torch.randn(1000, 64) * 5 + 3
+    y = torch.nn.functional.layer_norm(x, (64,), ln.weight, ln.bias)
+    assert float(y.norm(dim=-1).max()) <= _norm_bound(ln.weight, ln.bias, 64, torch.float32)
+
+    t = torch.zeros(4, 3, 2, 64)
+    assert _fold_scale(t, 0.125, "auto") is False
+    assert _fold_scale(t, 0.125, "folded") is True and _fold_scale(t, 0.125, "exact") is False
+    t.come_qk_bound = FOLD_SCALE_MAX_LOGIT / 0.125
+    assert _fold_scale(t, 0.125, "auto") is True
+    t.come_qk_bound = FOLD_SCALE_MAX_LOGIT / 0.125 * 1.01
+    assert _fold_scale(t, 0.125, "auto") is False
+    with pytest.raises(ValueError, match="scale_mode"):
+        _fold_scale(t, 0.125, "fast")

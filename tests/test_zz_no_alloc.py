@@ -22,21 +22,22 @@ def _inputs(lengths, seed, heads=HEADS):
     return qkv, bias, cu
 
 
-def _call(entry, qkv, bias, cu, max_len, work=None):
+def _call(entry, qkv, bias, cu, max_len, work=None, flags=0, out=None, lse=None):
     lib = _lib.load()
     total, _, heads, _ = qkv.shape
     q, k, v = qkv[:, 0], qkv[:, 1], qkv[:, 2]
-    out = torch.full((total, heads, D), float("nan"), dtype=qkv.dtype, device=DEV)
-    lse = torch.full((heads, total), float("nan"), dtype=torch.float32, device=DEV)
+    if out is None:
+        out = torch.full((total, heads, D), float("nan"), dtype=qkv.dtype, device=DEV)
+        lse = torch.full((heads, total), float("nan"), dtype=torch.float32, device=DEV)
     args = [q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.dtype_code(qkv.dtype),
             q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
             cu.data_ptr(), cu.numel() - 1, total, heads, D, bias.data_ptr(), max_len, 0.125,
             out.data_ptr(), out.stride(0), out.stride(1), lse.data_ptr()]
     stream = _lib.current_stream(qkv.device)
     if entry == "static":
-        status = lib.come_attn_varlen_fwd_static(*args, stream)
+        status = lib.come_attn_varlen_fwd_static(*args, flags, stream)
     else:
-        status = lib.come_attn_varlen_fwd_ws(*args, _lib.ptr(work), 0 if work is None else work.numel(), stream)
+        status = lib.come_attn_varlen_fwd_ws(*args, _lib.ptr(work), 0 if work is None else work.numel(), flags, stream)
     return status, out, lse
 
 
@@ -45,18 +46,29 @@ def test_static_matches_workspace_entry_twice_then_rejects_oversize():
     limit = lib.come_attn_static_work_bytes()
     assert limit == 64 << 20
     # first a 25 536-token segment, then a smaller one (12 288): both shapes use the key-split tail, i.e. the buffer
-    for seed, lengths in ((0, [25536]), (1, [12288])):
+    # (the second shape also with the other way of applying the scale: the flag travels through this entry point too)
+    for seed, lengths, flags in ((0, [25536], 0), (1, [12288], 0), (1, [12288], _lib.COME_ATTN_FOLD_SCALE)):
         need = lib.come_attn_work_bytes(len(lengths), sum(lengths), HEADS, max(lengths))
         assert 0 < need <= limit, "the shape must exercise the work buffer"
         qkv, bias, cu = _inputs(lengths, seed)
         work = torch.empty(need, dtype=torch.uint8, device=DEV)
-        st_ws, out_ws, lse_ws = _call("ws", qkv, bias, cu, max(lengths), work)
-        st, out, lse = _call("static", qkv, bias, cu, max(lengths))
+        st_ws, out_ws, lse_ws = _call("ws", qkv, bias, cu, max(lengths), work, flags)
+        st, out, lse = _call("static", qkv, bias, cu, max(lengths), None, flags)
         assert st_ws == 0 and st == 0, lib.come_last_error()
         torch.cuda.synchronize()
         assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
         assert torch.equal(out, out_ws)
         assert torch.equal(lse, lse_ws)
+        # the call itself takes no device memory: with its outputs already there, the free memory the driver
+        # reports and what torch's allocator holds are the same before and after a (warm) call
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        free_before, held_before = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
+        st, _, _ = _call("static", qkv, bias, cu, max(lengths), None, flags, out=out, lse=lse)
+        torch.cuda.synchronize()
+        assert st == 0
+        assert torch.cuda.mem_get_info()[0] == free_before and torch.cuda.memory_reserved() == held_before
+        assert torch.equal(out, out_ws)
         # and it differs from a launch that never used a buffer only by rounding (not by garbage from the array)
         st_plain, out_plain, _ = _call("ws", qkv, bias, cu, max(lengths), None)
         assert st_plain == 0
