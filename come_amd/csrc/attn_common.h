@@ -16,6 +16,7 @@ struct AttnArgs {
     int64_t total;
     int n_heads, n_mblocks, n_units;
     int rotate;                      // unit u starts its query blocks at position u (even block counts, see locate_block)
+    int out_wide;                    // out rows allow 16-byte stores (pointer and strides multiples of 16 bytes)
     float scale_log2;
     // key-split tail: the last nb_tail query blocks of every (segment, head) unit are computed by `splits`
     // workgroups each, every one over its share of the keys, into `work`; a second kernel combines them

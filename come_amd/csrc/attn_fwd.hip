@@ -656,6 +656,7 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
         }
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) m_run[qt] = m_row[qt] == -INFINITY ? 0.f : m_row[qt];
+        __syncthreads();                                        // the epilogue reuses the stages
     }
     if (idle) return;
 
@@ -683,14 +684,24 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
         return;
     }
 
-    // ---- epilogue: normalise, write O (and LSE)
+    // ---- epilogue: normalise, write O (and LSE).  In the accumulators a lane holds 8-byte pieces of one output row,
+    // 32 rows per store instruction; written like that, a wavefront's 32 stores touch 32 rows each and queue up in the
+    // memory pipeline for microseconds (2.5 of the 30 us of a workgroup on an 800-token segment).  Each wavefront
+    // therefore passes its two 32 x 64 tiles through 4 KiB of LDS (16-byte chunk c of row r at chunk c ^ (r & 7)) and
+    // stores whole 128-byte rows, eight rows per instruction.  The LDS comes from stages that nothing reads or fills
+    // any more: K of the last tile and of the two tiles staged behind it (landed before the loop's last barrier; only
+    // the stage after those is still being filled) and V of the tile before the last.
+    {
+        const int last = n_tiles - 1;
+        uint16_t *slot_base = wave_u < 2   ? &lds_k[last & 3][2048 * wave_u]
+                              : wave_u < 4 ? &lds_v[(last + 3) & 3][2048 * (wave_u - 2)]
+                              : wave_u < 6 ? &lds_k[(last + 1) & 3][2048 * (wave_u - 4)]
+                                           : &lds_k[(last + 2) & 3][2048 * (wave_u - 6)];
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
-        const float l_tot = sum_across_halves(l_run[qt]);
-        const float inv = 1.0f / l_tot;
-        const int row = q0 + (wave * 2 + qt) * 32 + r;
-        if (row < L) {
-            uint16_t *op = a.out + static_cast<int64_t>(seq_start + row) * a.o_rs + head * a.o_hs + 4 * h;
+        for (int qt = 0; qt < 2; ++qt) {
+            const float l_tot = sum_across_halves(l_run[qt]);
+            const float inv = 1.0f / l_tot;
+            const int row = q0 + (wave * 2 + qt) * 32 + r;
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
@@ -698,11 +709,27 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
                     u32x2 w;
                     w[0] = E::pack2(o_acc[qt][dt][4 * g] * inv, o_acc[qt][dt][4 * g + 1] * inv);
                     w[1] = E::pack2(o_acc[qt][dt][4 * g + 2] * inv, o_acc[qt][dt][4 * g + 3] * inv);
-                    *reinterpret_cast<u32x2 *>(op + 32 * dt + 8 * g) = w;
+                    *reinterpret_cast<u32x2 *>(slot_base + r * 64 + (((4 * dt + g) ^ (r & 7)) << 3) + 4 * h) = w;
                 }
-            if (h == 0 && a.lse)
+            if (row < L && h == 0 && a.lse)
                 a.lse[static_cast<int64_t>(head) * a.total + seq_start + row] =
                     (m_run[qt] + __log2f(l_tot)) * 0.6931471805599453f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int tr = 8 * i + (lane >> 3);                        // row of the tile, 8 lanes per row
+                const int c = (lane & 7) ^ (tr & 7);                       // the chunk this lane finds at position lane % 8
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(slot_base + tr * 64 + ((lane & 7) << 3));
+                const int orow = q0 + (wave * 2 + qt) * 32 + tr;
+                if (orow < L) {
+                    uint16_t *op = a.out + static_cast<int64_t>(seq_start + orow) * a.o_rs + head * a.o_hs + 8 * c;
+                    if (a.out_wide) {
+                        *reinterpret_cast<u32x4 *>(op) = v;
+                    } else {
+                        *reinterpret_cast<u32x2 *>(op) = u32x2{v[0], v[1]};
+                        *reinterpret_cast<u32x2 *>(op + 4) = u32x2{v[2], v[3]};
+                    }
+                }
+            }
         }
     }
 }
@@ -948,6 +975,7 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
     a.scale_log2 = softmax_scale * 1.4426950408889634f;
     a.n_units = static_cast<int>(n_seq * n_heads);
     a.rotate = (!wide && a.n_mblocks % 2 == 0) ? 1 : 0;
+    a.out_wide = (o_row_stride % 8 == 0 && o_head_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) ? 1 : 0;
     a.nb_tail = plan.nb_tail;
     a.splits = plan.splits;
     a.work = static_cast<float *>(work);
