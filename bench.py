@@ -52,7 +52,9 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the merge / unmerge microbenchmarks")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
-    ap.add_argument("--only", choices=["attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "prologue", "copy", "exact", "folded", "widths", "select", "e2e", "stress", "stress_e2e", "frame"], default=None,
+    ap.add_argument("--scale-mode", choices=["auto", "exact", "folded"], default="auto",
+                    help="with --only frame / stress_frames: how softmax_scale is applied (one kernel per profiler run)")
+    ap.add_argument("--only", choices=["stress_frames", "attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "prologue", "copy", "exact", "folded", "widths", "select", "e2e", "stress", "stress_e2e", "frame"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -275,6 +277,68 @@ def bench_merge_unmerge(device, iters=200, warmup=20):
     }
 
 
+def bench_merge_operator(device, w, iters=200, warmup=20):
+    """The confidence-guided merge as a caller of ``co_me_cuext.co_me_select_merge_2d`` sees it: selection + plan,
+    the 4-byte device-to-host read of the packed row count that sizes the output, the allocations from torch's caching
+    allocator and the gather-mean, per call on the wall clock (the read makes every call synchronous), over the
+    rotating token sets of the microbenchmark.  Next to it the reference-shaped chain of two calls
+    (``co_me_select_windows`` then ``co_me_token_merge_2d_cuda``), which plans in a launch of its own."""
+    import torch
+    from come_amd.cuda_extension import co_me_cuext
+
+    tokens, conf, sets = w["tokens"], w["conf"], len(w["tokens"])
+    frames, H, W = w["frames"], 37, 37
+    state = {"i": 0}
+
+    def fused():
+        i = state["i"] = (state["i"] + 1) % sets
+        return co_me_cuext.co_me_select_merge_2d(tokens[i], conf, 1, 5, 3, 3, H, W, w["ratio"])
+
+    def two_calls():
+        i = state["i"] = (state["i"] + 1) % sets
+        mask = co_me_cuext.co_me_select_windows(conf, 1, 3, 3, w["ratio"])
+        return co_me_cuext.co_me_token_merge_2d_cuda(tokens[i], 5, 3, 3, H, W, mask, index_dtype=torch.int32,
+                                                     count_dtype=torch.int32)
+
+    def median_us(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(iters):
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e6)
+        return sorted(times)[len(times) // 2]
+
+    fused_us, two_us = median_us(fused), median_us(two_calls)
+    assert fused()[0].shape[0] == w["P"]
+    return {"co_me_select_merge_2d_us": round(fused_us, 1),
+            "GBs": round(w["merge_bytes"] / (fused_us * 1e-6) / 1e9, 1),
+            "frac": round(w["merge_bytes"] / (fused_us * 1e-6) / 1e9 / PEAK_HBM_GBS, 4),
+            "select_then_merge_calls_us": round(two_us, 1), "statistic": "median wall time per call, synchronised",
+            "includes": "selection + plan launch, 4-byte read of the packed row count, output allocation, merge launch"}
+
+
+def bench_write_floor(device, nbytes, iters=200, warmup=20):
+    """A plain fill of ``nbytes`` over rotating buffers: what this part sustains for a stream of writes of the size
+    of the unmerge's output, the dominant stream of that kernel."""
+    import torch
+
+    sets = max(8, -(-320_000_000 // nbytes))
+    bufs = [torch.empty(nbytes // 4, dtype=torch.int32, device=device) for _ in range(sets)]
+    state = {"i": 0}
+
+    def fill():
+        i = state["i"] = (state["i"] + 1) % sets
+        bufs[i].fill_(1)
+
+    _, ms = time_loop(fill, iters, warmup)
+    return {"bytes": nbytes, "us_per_call": round(ms / iters * 1e3, 2), "GBs": round(nbytes / (ms / iters * 1e-3) / 1e9, 1),
+            "kernel": "torch fill_", "rotating_buffer_sets": sets}
+
+
 def bench_merge_caller_dtypes(device, iters=200, warmup=20):
     """The two other tensors the fused aggregator of the reference merges (vggt/fused.py:126-129): the fp32 residual
     stream [frames, N, 1024] and the bf16 positions [frames, N, 2] (element-wise kernels: rows of 4 bytes)."""
@@ -477,8 +541,9 @@ def bench_qk_prologue(device, rows=(25536, 43968), iters=200, warmup=20):
     return out
 
 
-def bench_frame_attention(device, w):
-    """Frame-mode attention of the headline workload's first sequence: 32 segments of about 798 tokens."""
+def bench_frame_attention(device, w, only_mode=None):
+    """Frame-mode attention of the headline workload's first sequence: 32 segments of about 798 tokens.
+    ``only_mode``: time that scale mode alone (profiler runs)."""
     import torch
 
     counts = packed_counts(32, 144, 5, 73, 2304, torch.Generator().manual_seed(0))
@@ -488,6 +553,10 @@ def bench_frame_attention(device, w):
     assert len(lens) == 32 and sum(lens) == counts.numel()
     # launches of 0.1 - 0.2 ms: the figure settles only after some tens of milliseconds under load (142 us with 10
     # warm-up launches, 119 us from about 200 on), hence the long warm-up
+    if only_mode is not None:
+        ms, tflops, flops = attention_case(device, lens, counts, steps=200, warmup=300, scale_mode=only_mode)
+        return {"scale_mode": only_mode, "us_per_call": round(ms * 1e3, 1), "value": round(tflops, 1), "unit": "TFLOP/s",
+                "algorithmic_flops": flops, "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
     ms, tflops, flops = attention_case(device, lens, counts, steps=200, warmup=300)
     ms_f, tflops_f, _ = attention_case(device, lens, counts, steps=200, warmup=100, scale_mode="folded")
     return {"workload": "frame attention: 32 segments of %d..%d packed tokens (same tokens as the headline sequence 0)"
@@ -497,9 +566,10 @@ def bench_frame_attention(device, w):
                              "frac": round(tflops_f / PEAK_BF16_TFLOPS, 4)}}
 
 
-def bench_stress(device):
+def bench_stress(device, frames_only_mode=None):
     """Long-sequence stress configuration at kernel level: 128 frames of 37x28 patches + 5 specials (133 248
-    tokens), 3x3 merge at ratio 0.75 with per-frame jitter +-0.1."""
+    tokens), 3x3 merge at ratio 0.75 with per-frame jitter +-0.1.  ``frames_only_mode``: only the frame attention of
+    that workload, in that scale mode (profiler runs)."""
     import torch
 
     w = merge_workload(device, ratio=0.75, sets=4, frames=128, H=37, W=28, jitter=0.1)   # 4 x 102 MB of packed rows
@@ -519,6 +589,10 @@ def bench_stress(device):
     P = w["P"]
     del w
     torch.cuda.empty_cache()
+    if frames_only_mode is not None:
+        ms, tflops, flops = attention_case(device, frame_lens, counts, steps=200, warmup=300, scale_mode=frames_only_mode)
+        return {"workload": res["workload"], "scale_mode": frames_only_mode, "us_per_call": round(ms * 1e3, 1),
+                "TFLOPs": round(tflops, 1), "algorithmic_flops": flops, "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
     ms, tflops, flops = attention_case(device, frame_lens, counts, steps=200, warmup=300)
     ms_f, tflops_f, _ = attention_case(device, frame_lens, counts, steps=200, warmup=100, scale_mode="folded")
     res["frame_attention"] = {"us_per_call": round(ms * 1e3, 1), "TFLOPs": round(tflops, 1), "algorithmic_flops": flops,
@@ -711,7 +785,11 @@ def main():
         if args.only == "stress":
             print(json.dumps({"only": "stress", **bench_stress(device)}))
         elif args.only == "frame":
-            print(json.dumps({"only": "frame", **bench_frame_attention(device, None)}))
+            print(json.dumps({"only": "frame", **bench_frame_attention(
+                device, None, None if args.scale_mode == "auto" else args.scale_mode)}))
+        elif args.only == "stress_frames":
+            print(json.dumps({"only": "stress_frames", **bench_stress(
+                device, "exact" if args.scale_mode == "auto" else args.scale_mode)}))
         elif args.only == "e2e":
             print(json.dumps({"only": "e2e", **bench_e2e(device, reps=max(1, args.steps))}))
         elif args.only == "stress_e2e":                          # seconds per forward: not part of the default run
@@ -794,6 +872,8 @@ def main():
     if not args.no_other:
         mw, other = bench_merge_unmerge(device)
         result["other"] = other
+        other["merge"]["operator"] = bench_merge_operator(device, mw)
+        other["unmerge"]["write_floor"] = bench_write_floor(device, mw["frames"] * mw["N"] * mw["C"] * 2)
         other["unmerge_pair"] = bench_unmerge_pair(device, mw)
         other["library_gemm_reference"] = bench_gemm_reference(device)
         other["merge_other_ratios"] = bench_merge_ratios(device)

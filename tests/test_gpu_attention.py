@@ -399,6 +399,32 @@ def test_strided_views_and_separate_tensors():
     _compare(out2, ref)
 
 
+@pytest.mark.parametrize("pad,offset", [(4, 0), (8, 4), (12, 0)], ids=["stride68", "stride72+4", "stride76"])
+def test_output_views_that_do_not_allow_16_byte_stores(pad, offset):
+    """``out_`` may be a view whose head stride or start is only a multiple of 8 bytes: the kernel then writes its
+    rows in 8-byte pieces.  Same bits as into a contiguous output; the padding of the view stays untouched."""
+    lens, H = [300, 77, 513], 3
+    P = sum(lens)
+    g = torch.Generator().manual_seed(pad)
+    qkv = torch.randn(P, 3, H, 64, generator=g).bfloat16().to(DEV)
+    bias = torch.where(torch.rand(P, generator=g) < 0.3, math.log(9.0), 0.0).bfloat16().to(DEV)
+    cu = _cu(lens).to(DEV)
+    q, k, v = qkv.unbind(1)
+    call = lambda out_: flash_attn_fwd_cuda.varlen_fwd_w_perkey_bias(
+        q, k, v, out_, cu, cu, None, None, None, None, bias, max(lens), max(lens), 0.0, 0.125, False, False, -1, -1,
+        0.0, False, None)[0]
+    want = call(None)
+    wide = torch.full((P, H, 64 + pad), 7.0, dtype=torch.bfloat16, device=DEV)
+    view = wide[:, :, offset:offset + 64]
+    assert view.stride(1) % 8 != 0 or view.data_ptr() % 16 != 0
+    got = call(view)
+    assert got.data_ptr() == view.data_ptr()
+    assert torch.equal(got, want)
+    untouched = torch.ones(64 + pad, dtype=torch.bool)
+    untouched[offset:offset + 64] = False
+    assert bool((wide[:, :, untouched.to(DEV)] == 7.0).all())
+
+
 def test_max_seqlen_helper_and_empty_segment():
     lens = [40, 0, 90]
     cu = _cu(lens).to(DEV)
