@@ -457,7 +457,7 @@ def bench_merge_ratios(device, iters=200, warmup=20):
     return out
 
 
-def attention_case(device, lens, counts, steps, warmup, H=16, D=64, scale_mode="auto"):
+def attention_case(device, lens, counts, steps, warmup, H=16, D=64, scale_mode="auto", work_queue=False):
     """Times the biased attention on packed segments ``lens`` with per-key counts; returns (ms, TFLOP/s)."""
     import torch
     from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
@@ -473,7 +473,8 @@ def attention_case(device, lens, counts, steps, warmup, H=16, D=64, scale_mode="
     max_len = max(lens)
     _, ms = time_loop(lambda: flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu, max_len, perkey_bias=bias,
                                                                              softmax_scale=0.125,
-                                                                             scale_mode=scale_mode), steps, warmup)
+                                                                             scale_mode=scale_mode,
+                                                                             work_queue=work_queue), steps, warmup)
     flops = sum(4.0 * n * n * D * H for n in lens)
     return ms / steps, flops / (ms / steps * 1e-3) / 1e12, flops
 
@@ -559,11 +560,15 @@ def bench_frame_attention(device, w, only_mode=None):
                 "algorithmic_flops": flops, "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
     ms, tflops, flops = attention_case(device, lens, counts, steps=200, warmup=300)
     ms_f, tflops_f, _ = attention_case(device, lens, counts, steps=200, warmup=100, scale_mode="folded")
+    ms_q, tflops_q, _ = attention_case(device, lens, counts, steps=200, warmup=100, work_queue=True)
     return {"workload": "frame attention: 32 segments of %d..%d packed tokens (same tokens as the headline sequence 0)"
                         % (min(lens), max(lens)), "us_per_call": round(ms * 1e3, 1), "value": round(tflops, 1),
             "unit": "TFLOP/s", "algorithmic_flops": flops, "frac": round(tflops / PEAK_BF16_TFLOPS, 4),
             "folded_scale": {"us_per_call": round(ms_f * 1e3, 1), "value": round(tflops_f, 1),
-                             "frac": round(tflops_f / PEAK_BF16_TFLOPS, 4)}}
+                             "frac": round(tflops_f / PEAK_BF16_TFLOPS, 4)},
+            # the opt-in launch of resident workgroups fed from a device-side work list (list kernel included)
+            "work_queue": {"us_per_call": round(ms_q * 1e3, 1), "value": round(tflops_q, 1),
+                           "frac": round(tflops_q / PEAK_BF16_TFLOPS, 4)}}
 
 
 def bench_stress(device, frames_only_mode=None):
@@ -595,10 +600,13 @@ def bench_stress(device, frames_only_mode=None):
                 "TFLOPs": round(tflops, 1), "algorithmic_flops": flops, "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}
     ms, tflops, flops = attention_case(device, frame_lens, counts, steps=200, warmup=300)
     ms_f, tflops_f, _ = attention_case(device, frame_lens, counts, steps=200, warmup=100, scale_mode="folded")
+    ms_q, tflops_q, _ = attention_case(device, frame_lens, counts, steps=200, warmup=100, work_queue=True)
     res["frame_attention"] = {"us_per_call": round(ms * 1e3, 1), "TFLOPs": round(tflops, 1), "algorithmic_flops": flops,
                               "frac": round(tflops / PEAK_BF16_TFLOPS, 4),
                               "folded_scale": {"us_per_call": round(ms_f * 1e3, 1), "TFLOPs": round(tflops_f, 1),
-                                               "frac": round(tflops_f / PEAK_BF16_TFLOPS, 4)}}
+                                               "frac": round(tflops_f / PEAK_BF16_TFLOPS, 4)},
+                              "work_queue": {"us_per_call": round(ms_q * 1e3, 1), "TFLOPs": round(tflops_q, 1),
+                                             "frac": round(tflops_q / PEAK_BF16_TFLOPS, 4)}}
     ms, tflops, flops = attention_case(device, [P], counts, steps=5, warmup=2)
     res["global_attention"] = {"ms_per_call": round(ms, 3), "TFLOPs": round(tflops, 1), "algorithmic_flops": flops,
                                "frac": round(tflops / PEAK_BF16_TFLOPS, 4)}

@@ -17,7 +17,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("COME_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libcome_hip.so")
 
 COME_F32, COME_F16, COME_BF16 = 0, 1, 2
-COME_ATTN_FOLD_SCALE = 1          # bit of the attention entry points' `flags`
+COME_ATTN_FOLD_SCALE, COME_ATTN_WORK_QUEUE = 1, 2          # bits of the attention entry points' `flags`
 
 _DTYPE_CODE = {torch.float32: COME_F32, torch.float16: COME_F16, torch.bfloat16: COME_BF16}
 
@@ -44,6 +44,7 @@ SIGNATURES = {
                                     _ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _f32,
                                     _ptr, _i64, _i64, _ptr, _int, _ptr]),
     "come_attn_work_bytes": (_i64, [_i64, _i64, _i64, _i64]),
+    "come_attn_queue_bytes": (_i64, [_i64, _i64, _i64]),
     "come_attn_varlen_fwd_ws": (_int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64,
                                        _ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _f32,
                                        _ptr, _i64, _i64, _ptr, _ptr, _i64, _int, _ptr]),

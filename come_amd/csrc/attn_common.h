@@ -23,6 +23,10 @@ struct AttnArgs {
     int nb_tail, splits;
     int64_t n_full_wg;               // workgroups in front of the split ones
     float *work;
+    // work queue of a launch of resident workgroups: 8 claim counters (one per class of workgroups, blockIdx.x % 8),
+    // 8 item counts, then 8 lists of queue_cap entries (unit << 8 | query block)
+    uint32_t *queue;
+    int queue_cap;
 };
 
 namespace {

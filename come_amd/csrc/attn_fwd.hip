@@ -98,6 +98,9 @@ __device__ inline bool locate_block(const AttnArgs &a, int &mblk, int &head, int
 // subtraction, one exp2, half a pack and half a dot per score on the vector ALU and nothing else.
 // -------------------------------------------------------------------------------------
 constexpr int kStages = 4;
+// Launches whose segments are at most this long walk their work items in resident workgroups (PERSIST below): a few
+// query blocks per (segment, head) unit, so a fixed share of the item list per workgroup is a balanced share.
+constexpr int64_t kPersistMaxSeqlen = 2048;
 
 // Range of the probabilities relative to the reference point of their row.  They are stored in the 16-bit type of
 // the inputs: bf16 has the exponent range of fp32, fp16 reaches only 65504 and loses precision below 2^-14.
@@ -119,11 +122,20 @@ template <> struct Range<COME_F16> {
     static constexpr float kHardLimit = 32768.f;           // one probability near 65504 (where the conversion saturates)
 };
 
-template <int DT, int NW, bool EXACT>
-__global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a) {
+//
+// PERSIST (short segments, 4 wavefronts): the launch has two workgroups per CU and every workgroup walks a list of work
+// items - (segment, head, 256-query block) - of its own: item g, g + G, g + 2 G, ... of the launch's G workgroups.  The
+// K / V / bias ring does not stop at the end of an item: the last iterations of an item stage the first tiles of the
+// next one (other segment, other head), its Q rows are requested as soon as the last scores of the current item have
+// been issued, and arrive while the current item is normalised and written.  What a short segment otherwise pays per
+// workgroup - the chain of dependent latencies from the segment offsets to the first staged tiles, and the launch
+// of a new workgroup - is paid once per workgroup instead of once per item.
+template <int DT, int NW, bool EXACT, bool PERSIST>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_fwd_pipe_kernel(const AttnArgs a) {
     using E = Elem<DT>;
     constexpr float kSumLimit = Range<DT>::kSumLimit;
     static_assert(NW == 4 || NW == 8, "4 or 8 wavefronts per workgroup");
+    static_assert(!PERSIST || NW == 4, "the item loop exists for 256-query workgroups");
     constexpr int kBlockM = 64 * NW;           // queries per workgroup
     constexpr int kThreads = 64 * NW;
     constexpr int kDma = 8 / NW;               // direct loads per wavefront for one K (or V) tile
@@ -137,27 +149,62 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     __shared__ __attribute__((aligned(256))) uint32_t lds_braw[kStages][kBlockN];   // raw bias words as loaded
     __shared__ float lds_ref[NW];                                                   // prologue: reference point per wavefront
 
-    int mblk, head, seq, tail, ks;
-    if (!locate_block(a, mblk, head, seq, tail, ks)) return;
-    int seq_start, L;
-    segment_of(a, seq, seq_start, L);
-    const int n_qblocks = (L + kBlockM - 1) / kBlockM;
-    if (tail >= 0) {
-        mblk = n_qblocks - a.nb_tail + tail;          // split workgroup: one of the unit's last query blocks
-        if (mblk < 0) return;
-    } else if (a.splits > 1 && mblk >= n_qblocks - a.nb_tail) {
-        return;                                       // left to the split workgroups (or beyond the segment)
-    }
-    const int q0 = mblk * kBlockM;
-    if (q0 >= L) return;
-    // keys of this workgroup: all tiles, or share ks of them
-    const int all_tiles = (L + kBlockN - 1) / kBlockN;
-    const int tile_base = tail >= 0 ? static_cast<int>(static_cast<int64_t>(ks) * all_tiles / a.splits) : 0;
-    const int tile_end = tail >= 0 ? static_cast<int>(static_cast<int64_t>(ks + 1) * all_tiles / a.splits) : all_tiles;
+    // ---- the work item (wave-uniform): rows seq_start .. + L of the packed tensors, one head, queries q0 .. of the
+    // segment; key tiles tile_base .. tile_base + n_tiles (all tiles of the segment unless the workgroup computes a
+    // key share into `piece`).  nx_*: PERSIST, the item after it.
+    int seq_start = 0, L = 0, head = 0, q0 = 0, tile_base = 0, n_tiles = 0;
     float *piece = nullptr;
-    if (tail >= 0) {
-        const int64_t index = (static_cast<int64_t>(seq * a.n_heads + head) * a.nb_tail + tail) * a.splits + ks;
-        piece = a.work + index * (kBlockM * (kHeadDim + kPieceExtra));
+    int nx_seq_start = 0, nx_L = 0, nx_head = 0, nx_q0 = 0;
+    bool has_next = false;
+    // PERSIST: the workgroups of class c = blockIdx.x % 8 (dispatched to XCD c) share list c of the queue, which
+    // attn_items_kernel filled with the query blocks of the units u = c mod 8, block after block and unit after unit, so
+    // that the workgroups resident on one XCD work on the blocks of the same few units at the same time and find
+    // their K / V in that L2.  A workgroup's first two items are fixed by its index; every further one is claimed from
+    // the class counter, two items ahead: the claim is issued at the top of an item, published to the workgroup on the
+    // last barrier of its key loop, and the item it names is looked up while the current item is written.
+    // (The two workgroups of a CU do not run at the same pace: the one dispatched first wins every arbitration for the
+    // matrix pipe and runs its tiles about 1.4 times as fast, for the whole launch.  A fixed share per workgroup would
+    // leave the CUs half empty at the end; with the queue the faster one simply takes more items.)
+    __shared__ uint32_t lds_claim;
+    const uint32_t cls = blockIdx.x & 7u, per_cls = gridDim.x >> 3;
+    const uint32_t *item_list = PERSIST ? a.queue + 16 + static_cast<size_t>(cls) * a.queue_cap : nullptr;
+    uint32_t n_items = 0;
+    int aa_seq_start = 0, aa_L = 0, aa_head = 0, aa_q0 = 0;          // the item after the next one
+    auto decode_item = [&](uint32_t t, int &o_start, int &o_len, int &o_head, int &o_q0) __attribute__((always_inline)) {
+        const uint32_t entry = item_list[t];
+        const uint32_t unit = entry >> 8;
+        segment_of(a, static_cast<int>(unit / static_cast<uint32_t>(a.n_heads)), o_start, o_len);
+        o_head = static_cast<int>(unit % static_cast<uint32_t>(a.n_heads));
+        o_q0 = static_cast<int>(entry & 255u) * kBlockM;
+    };
+    if constexpr (PERSIST) {
+        n_items = a.queue[8 + cls];
+        const uint32_t t0 = blockIdx.x >> 3, t1 = t0 + per_cls;
+        if (t0 >= n_items) return;
+        decode_item(t0, seq_start, L, head, q0);
+        has_next = t1 < n_items;
+        if (has_next) decode_item(t1, nx_seq_start, nx_L, nx_head, nx_q0);
+    } else {
+        int mblk, seq, tail, ks;
+        if (!locate_block(a, mblk, head, seq, tail, ks)) return;
+        segment_of(a, seq, seq_start, L);
+        const int n_qblocks = (L + kBlockM - 1) / kBlockM;
+        if (tail >= 0) {
+            mblk = n_qblocks - a.nb_tail + tail;          // split workgroup: one of the unit's last query blocks
+            if (mblk < 0) return;
+        } else if (a.splits > 1 && mblk >= n_qblocks - a.nb_tail) {
+            return;                                       // left to the split workgroups (or beyond the segment)
+        }
+        q0 = mblk * kBlockM;
+        if (q0 >= L) return;
+        // keys of this workgroup: all tiles, or share ks of them
+        const int all_tiles = (L + kBlockN - 1) / kBlockN;
+        tile_base = tail >= 0 ? static_cast<int>(static_cast<int64_t>(ks) * all_tiles / a.splits) : 0;
+        n_tiles = (tail >= 0 ? static_cast<int>(static_cast<int64_t>(ks + 1) * all_tiles / a.splits) : all_tiles) - tile_base;
+        if (tail >= 0) {
+            const int64_t index = (static_cast<int64_t>(seq * a.n_heads + head) * a.nb_tail + tail) * a.splits + ks;
+            piece = a.work + index * (kBlockM * (kHeadDim + kPieceExtra));
+        }
     }
 
     const int tid = threadIdx.x;
@@ -171,34 +218,51 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     // the MFMA unscaled and c is applied in fp32 in front of the exponential, as the reference applies it
     // (softmax.h:76-88).  Otherwise scaled by c here and rounded back to 16 bit.
     u32x4 qf[2][4];
+    // (tl: the thread index, passed in so that the item loop can hand over a copy the compiler knows nothing about -
+    // otherwise every address term that depends on the lane alone is kept in a register across the whole loop)
+    auto load_q = [&](int tl, int start, int len, int hd, int first) __attribute__((always_inline)) {
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
-        const int row = q0 + (wave * 2 + qt) * 32 + r;
-        const uint16_t *qp = a.q + static_cast<int64_t>(seq_start + min(row, L - 1)) * a.q_rs + head * a.q_hs + 8 * h;
+        for (int qt = 0; qt < 2; ++qt) {
+            const int row = first + ((tl >> 6) * 2 + qt) * 32 + (tl & 31);
+            const uint16_t *qp = a.q + static_cast<int64_t>(start + min(row, len - 1)) * a.q_rs + hd * a.q_hs + 8 * ((tl >> 5) & 1);
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            const u32x4 raw = *reinterpret_cast<const u32x4 *>(qp + 16 * ks);
-            if (EXACT) {
-                qf[qt][ks] = raw;
-            } else {
-#pragma unroll
-                for (int w = 0; w < 4; ++w)
-                    qf[qt][ks][w] = E::pack2(E::to_f32(static_cast<uint16_t>(raw[w] & 0xffffu)) * a.scale_log2,
-                                             E::to_f32(static_cast<uint16_t>(raw[w] >> 16)) * a.scale_log2);
-            }
+            for (int ks = 0; ks < 4; ++ks) qf[qt][ks] = *reinterpret_cast<const u32x4 *>(qp + 16 * ks);
         }
+    };
+    auto scale_q = [&]() __attribute__((always_inline)) {
+        if (EXACT) return;
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const uint32_t raw = qf[qt][ks][w];
+                    qf[qt][ks][w] = E::pack2(E::to_f32(static_cast<uint16_t>(raw & 0xffffu)) * a.scale_log2,
+                                             E::to_f32(static_cast<uint16_t>(raw >> 16)) * a.scale_log2);
+                }
+    };
+    if constexpr (!PERSIST) {
+        load_q(tid, seq_start, L, head, q0);
+        scale_q();
     }
     // ---- global -> LDS staging.  Wavefront w fills rows 16 w .. 16 w + 15 of a tile with two direct
     // loads; lane l of load i brings row 8 (2 w + i) + l / 8, slot l % 8.  A key index beyond the segment
     // is redirected to its last key (finite data); such keys get a bias term of -inf, so their
     // probabilities are exactly 0 and neither their K nor their V row can reach the output.
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const char *k_seg = reinterpret_cast<const char *>(a.k + static_cast<int64_t>(seq_start) * a.k_rs + head * a.k_hs);
-    const char *v_seg = reinterpret_cast<const char *>(a.v + static_cast<int64_t>(seq_start) * a.v_rs + head * a.v_hs);
-    // bias of the segment as bytes from a 4-byte aligned base: b_mis is the misalignment of its first key
-    const uintptr_t b_addr = reinterpret_cast<uintptr_t>(a.bias) + 2u * static_cast<uintptr_t>(seq_start);
-    const char *b_seg = a.bias ? reinterpret_cast<const char *>(b_addr & ~static_cast<uintptr_t>(3)) : nullptr;
-    const uint32_t b_mis = static_cast<uint32_t>(b_addr & 3);
+    // K, V of the item's segment and head; its bias as bytes from a 4-byte aligned base (b_mis: the misalignment of
+    // the first key).  nx_*: the same for the next item.
+    const char *k_seg, *v_seg, *b_seg, *nx_k_seg = nullptr, *nx_v_seg = nullptr, *nx_b_seg = nullptr;
+    uint32_t b_mis, nx_b_mis = 0;
+    auto segment_pointers = [&](int start, int hd, const char *&ks, const char *&vs, const char *&bs, uint32_t &mis) __attribute__((always_inline)) {
+        ks = reinterpret_cast<const char *>(a.k + static_cast<int64_t>(start) * a.k_rs + hd * a.k_hs);
+        vs = reinterpret_cast<const char *>(a.v + static_cast<int64_t>(start) * a.v_rs + hd * a.v_hs);
+        const uintptr_t b_addr = reinterpret_cast<uintptr_t>(a.bias) + 2u * static_cast<uintptr_t>(start);
+        bs = a.bias ? reinterpret_cast<const char *>(b_addr & ~static_cast<uintptr_t>(3)) : nullptr;
+        mis = static_cast<uint32_t>(b_addr & 3);
+    };
+    segment_pointers(seq_start, head, k_seg, v_seg, b_seg, b_mis);
     const uint32_t k_rs_b = static_cast<uint32_t>(a.k_rs) * 2u, v_rs_b = static_cast<uint32_t>(a.v_rs) * 2u;
     uint32_t k_goff[kDma], v_goff[kDma], k_chunk[kDma], v_chunk[kDma];
     int st_row[kDma];
@@ -210,40 +274,53 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
         k_goff[i] = static_cast<uint32_t>(st_row[i]) * k_rs_b + k_chunk[i];
         v_goff[i] = static_cast<uint32_t>(st_row[i]) * v_rs_b + v_chunk[i];
     }
-    const uint32_t k_last = static_cast<uint32_t>(L - 1) * k_rs_b, v_last = static_cast<uint32_t>(L - 1) * v_rs_b;
     const uint32_t k_tile_step = static_cast<uint32_t>(kBlockN) * k_rs_b, v_tile_step = static_cast<uint32_t>(kBlockN) * v_rs_b;
 
+    // rel_tile counts from the item's first tile; PERSIST: tiles behind the item's last one are the first tiles of the
+    // next item (the ring runs on)
     auto stage_k = [&](int rel_tile, int buf) __attribute__((always_inline)) {
-        const int tile = tile_base + rel_tile;
+        const bool own = !PERSIST || rel_tile < n_tiles;                            // wave-uniform, like all of these
+        const char *base = own ? k_seg : nx_k_seg;
+        const int len = own ? L : nx_L;
+        const int tile = tile_base + (own ? rel_tile : rel_tile - n_tiles);
         const int n0 = tile * kBlockN;
-        const uint32_t tile_off = static_cast<uint32_t>(tile) * k_tile_step;         // wave-uniform
-        const bool full = n0 + kBlockN <= L;                                        // wave-uniform
+        const uint32_t tile_off = static_cast<uint32_t>(tile) * k_tile_step;
+        const uint32_t last = static_cast<uint32_t>(len - 1) * k_rs_b;
+        const bool full = n0 + kBlockN <= len;
 #pragma unroll
         for (int i = 0; i < kDma; ++i) {
             uint32_t off = tile_off + k_goff[i];
-            if (!full) off = n0 + st_row[i] < L ? off : k_last + k_chunk[i];
-            dma_b128(k_seg, off, lds_address(&lds_k[buf][(kDma * wave_u + i) * 512]));
+            if (!full) off = n0 + st_row[i] < len ? off : last + k_chunk[i];
+            dma_b128(base, off, lds_address(&lds_k[buf][(kDma * wave_u + i) * 512]));
         }
     };
     // raw bias of the 64 keys of a tile: wavefront 0 brings the aligned 32-bit word that holds each key's
     // 16-bit bias; it is converted to a float two iterations later (commit_bias)
     auto load_bias = [&](int rel_tile, int buf) __attribute__((always_inline)) {
-        const int tile = tile_base + rel_tile;
-        if (wave_u == 0 && b_seg) {
-            const uint32_t key = static_cast<uint32_t>(min(tile * kBlockN + lane, L - 1));
-            dma_b32(b_seg, ((b_mis + 2u * key) & ~3u), lds_address(&lds_braw[buf][0]));
+        const bool own = !PERSIST || rel_tile < n_tiles;
+        const char *base = own ? b_seg : nx_b_seg;
+        const int len = own ? L : nx_L;
+        const uint32_t mis = own ? b_mis : nx_b_mis;
+        const int tile = tile_base + (own ? rel_tile : rel_tile - n_tiles);
+        if (wave_u == 0 && a.bias) {
+            const uint32_t key = static_cast<uint32_t>(min(tile * kBlockN + lane, len - 1));
+            dma_b32(base, ((mis + 2u * key) & ~3u), lds_address(&lds_braw[buf][0]));
         }
     };
     auto stage_v = [&](int rel_tile, int buf) __attribute__((always_inline)) {
-        const int tile = tile_base + rel_tile;
+        const bool own = !PERSIST || rel_tile < n_tiles;
+        const char *base = own ? v_seg : nx_v_seg;
+        const int len = own ? L : nx_L;
+        const int tile = tile_base + (own ? rel_tile : rel_tile - n_tiles);
         const int n0 = tile * kBlockN;
         const uint32_t tile_off = static_cast<uint32_t>(tile) * v_tile_step;
-        const bool full = n0 + kBlockN <= L;
+        const uint32_t last = static_cast<uint32_t>(len - 1) * v_rs_b;
+        const bool full = n0 + kBlockN <= len;
 #pragma unroll
         for (int i = 0; i < kDma; ++i) {
             uint32_t off = tile_off + v_goff[i];
-            if (!full) off = n0 + st_row[i] < L ? off : v_last + v_chunk[i];
-            dma_b128(v_seg, off, lds_address(&lds_v[buf][(kDma * wave_u + i) * 512]));
+            if (!full) off = n0 + st_row[i] < len ? off : last + v_chunk[i];
+            dma_b128(base, off, lds_address(&lds_v[buf][(kDma * wave_u + i) * 512]));
         }
     };
     // conversion of the raw bias of one tile, split in two so that the LDS read is in flight during a slot:
@@ -255,22 +332,27 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     float m_base = 0.f;           // reference point shared by the rows of the workgroup (uniform), log2 units
     uint32_t b_word = 0;
     auto peek_bias = [&](int buf) __attribute__((always_inline)) {
-        if (wave_u == 0 && b_seg) b_word = lds_braw[buf][lane];
+        if (wave_u == 0 && a.bias) b_word = lds_braw[buf][lane];
     };
+    // (a tile of the next item is converted against a reference point of 0: its own is not known yet)
     auto commit_bias = [&](int rel_tile, int buf) __attribute__((always_inline)) {
         if (wave_u == 0) {
-            const int key = (tile_base + rel_tile) * kBlockN + lane;
+            const bool own = !PERSIST || rel_tile < n_tiles;
+            const int len = own ? L : nx_L;
+            const uint32_t mis = own ? b_mis : nx_b_mis;
+            const float base = own ? m_base : 0.f;
+            const int key = (tile_base + (own ? rel_tile : rel_tile - n_tiles)) * kBlockN + lane;
             float bias = 0.f;
-            if (b_seg) {
-                const uint32_t at = b_mis + 2u * static_cast<uint32_t>(min(key, L - 1));
+            if (a.bias) {
+                const uint32_t at = mis + 2u * static_cast<uint32_t>(min(key, len - 1));
                 bias = E::to_f32(static_cast<uint16_t>((at & 2u) ? (b_word >> 16) : (b_word & 0xffffu)));
             }
-            lds_b[buf][lane] = key < L ? (bias * kLog2e - m_base) * unit : -INFINITY;
+            lds_b[buf][lane] = key < len ? (bias * kLog2e - base) * unit : -INFINITY;
         }
     };
     auto staged_wait = [&](bool with_bias_load) __attribute__((always_inline)) {
         // the direct loads issued in this iteration (K, V and, on wavefront 0, the bias) may stay in flight
-        if (with_bias_load && wave_u == 0 && b_seg) {
+        if (with_bias_load && wave_u == 0 && a.bias) {
             if (NW == 4) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
             else asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
         } else {
@@ -302,16 +384,6 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     float delta[2] = {0.f, 0.f};  // what the row's reference point differs from m_base by (0 for nearly all rows)
     bool has_delta = false;       // wave-uniform: some row of this wavefront has delta != 0
     float l_run[2] = {0.f, 0.f};  // per-lane partial row sum
-#pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
-        o_acc[qt][0] = zero16;
-        o_acc[qt][1] = zero16;
-#pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            p_frag[b][qt][0] = zero4();
-            p_frag[b][qt][1] = zero4();
-        }
-    }
 
     // scores of both query tiles against half-tile `half` of the K tile in `buf`, into buffer b: the accumulators
     // start from the LDS bias values of their keys and collect the four k-steps of (c Q) K^T
@@ -485,39 +557,91 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
         }
     };
 
-    // ---- prologue
-    const int n_tiles = tile_end - tile_base;
+    // ---- the item loop (a single pass unless PERSIST).  ring: stage of the item's tile 0 (the K / V / bias ring runs on
+    // from item to item); cold: nothing of this item has been staged yet (first item, or the one after a block that
+    // had to be computed again, which uses the stages for itself).
+    int ring = 0;
+    bool cold = true;
+    for (;;) {
+    int tl = tid;                            // this item's private copy of the thread index
+    if constexpr (PERSIST) asm volatile("" : "+v"(tl));
+    if constexpr (PERSIST) {
+        // at least kStages tiles per item, so that what an iteration stages ahead never reaches beyond the next item;
+        // tiles behind the end of the segment are masked like the tail of its last tile
+        n_tiles = max((L + kBlockN - 1) / kBlockN, kStages);
+        if (!has_next) {                     // staging ahead then re-reads the first tiles of this item
+            nx_seq_start = seq_start;
+            nx_L = L;
+            nx_head = head;
+        }
+        segment_pointers(nx_seq_start, nx_head, nx_k_seg, nx_v_seg, nx_b_seg, nx_b_mis);
+    }
+    uint32_t claim = 0;                      // (one lane) what the class counter hands out for the item after next
+    if constexpr (PERSIST) {
+        if (has_next && tl == 0)
+            claim = __hip_atomic_fetch_add(a.queue + cls, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     if (n_tiles <= 0) {                      // a key share without tiles (segment shorter than the split count)
-        for (int i = tid; i < kBlockM; i += kThreads) {
+        for (int i = tl; i < kBlockM; i += kThreads) {
             piece[kBlockM * kHeadDim + i] = -1e30f;               // reference point
             piece[kBlockM * (kHeadDim + 1) + i] = 0.f;            // row sum
         }
         return;
     }
-    {   // the last V stage stands in for "tile -1": zeros (its probabilities are zero as well)
-        u32x4 *z = reinterpret_cast<u32x4 *>(&lds_v[kStages - 1][0]);
-        for (int i = tid; i < kBlockN * kHeadDim / 8; i += kThreads) z[i] = zero4();
+    m_base = 0.f;
+    o_pending[0] = 1.f;
+    o_pending[1] = 1.f;
+    any_pending = false;
+    overflowed = false;
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+        o_acc[qt][0] = zero16;
+        o_acc[qt][1] = zero16;
+        l_run[qt] = 0.f;
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            p_frag[b][qt][0] = zero4();
+            p_frag[b][qt][1] = zero4();
+        }
     }
-    load_bias(0, 0);
-    load_bias(1, 1);
-    load_bias(2, 2);
-    load_bias(3, 3);
-    stage_k(0, 0);
-    stage_v(0, 0);
-    stage_k(1, 1);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    peek_bias(0);
-    commit_bias(0, 0);
-    peek_bias(1);
-    commit_bias(1, 1);
-    stage_k(2, 2);                     // tiles of iteration 1 start their flight
-    stage_v(1, 1);
-    staged_wait(false);                // everything but this last group has landed
+    if (cold) {
+        ring = 0;
+        if constexpr (PERSIST) {
+            __syncthreads();                   // (after a block that was computed again: nobody reads the stages any more)
+            load_q(tl, seq_start, L, head, q0);
+        }
+        {   // the last V stage stands in for "tile -1": zeros (its probabilities are zero as well)
+            u32x4 *z = reinterpret_cast<u32x4 *>(&lds_v[kStages - 1][0]);
+            for (int i = tl; i < kBlockN * kHeadDim / 8; i += kThreads) z[i] = zero4();
+        }
+        load_bias(0, 0);
+        load_bias(1, 1);
+        load_bias(2, 2);
+        load_bias(3, 3);
+        stage_k(0, 0);
+        stage_v(0, 0);
+        stage_k(1, 1);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        peek_bias(0);
+        commit_bias(0, 0);
+        peek_bias(1);
+        commit_bias(1, 1);
+        stage_k(2, 2);                     // tiles of iteration 1 start their flight
+        stage_v(1, 1);
+        staged_wait(false);                // everything but this last group has landed
+    } else {
+        // the previous item's last iterations staged K 0 .. 2, V 0 .. 1 and the bias of tiles 0 .. 3 of this one and
+        // converted the bias of tiles 0 and 1; its V tiles stand in for "tile -1" (finite, times zero probabilities);
+        // Q was requested behind its last iteration
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    if constexpr (PERSIST) scale_q();
     __syncthreads();
+    const int st0 = ring & 3, st1 = (ring + 1) & 3;
     // Reference points.  Every row looks at its maximum over the first 32 keys; m_base is the largest of them in
     // the workgroup and is folded into the bias values in LDS, so that in the steady state nothing is subtracted
     // per score.  A row whose own maximum is more than 2^kMaxGap below m_base keeps the difference as its delta.
-    score_mfma(0, 0, 0);               // bias values in LDS are still relative to 0: plain scores
+    score_mfma(0, st0, 0);             // bias values in LDS are still relative to 0: plain scores
     float row_max[2];
     float wave_max = -INFINITY;
 #pragma unroll
@@ -537,8 +661,8 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
 #pragma unroll
     for (int w = 1; w < NW; ++w) m_base = fmaxf(m_base, lds_ref[w]);
     if (wave_u == 0) {                 // tiles 0 and 1 were converted against a base of 0
-        lds_b[0][lane] -= m_base * unit;
-        lds_b[1][lane] -= m_base * unit;
+        lds_b[st0][lane] -= m_base * unit;
+        lds_b[st1][lane] -= m_base * unit;
     }
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
@@ -558,15 +682,16 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     const bool idle = q0 + wave_u * 64 >= L;
     if (idle) {
         for (int j = 0; j < n_tiles; ++j) {
-            stage_k(j + 3, (j + 3) & 3);
-            stage_v(j + 2, (j + 2) & 3);
+            stage_k(j + 3, (ring + j + 3) & 3);
+            stage_v(j + 2, (ring + j + 2) & 3);
             staged_wait(true);
             if (lane == 0) lds_ref[wave] = 0.f;
             __syncthreads();
         }
     } else {
         for (int j = 0; j < n_tiles; ++j) {
-            const int kb = j & 3, kb1 = (j + 1) & 3, kb2 = (j + 2) & 3, kb3 = (j + 3) & 3;   // stage of tile j, j+1, ..
+            const int t = ring + j;
+            const int kb = t & 3, kb1 = (t + 1) & 3, kb2 = (t + 2) & 3, kb3 = (t + 3) & 3;   // stage of tile j, j+1, ..
             load_bias(j + 4, kb);      // raw bias runs one more tile ahead (converted between the slots of iteration j+2)
             stage_k(j + 3, kb3);       // K(j+3) replaces K(j-1), V(j+2) replaces V(j-2): both idle since the
             stage_v(j + 2, kb2);       // last barrier; they are first read two barriers from now
@@ -582,15 +707,11 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
 
             staged_wait(true);         // loads issued one iteration ago have landed
             if (lane == 0) lds_ref[wave] = overflowed ? 1.f : 0.f;      // (read behind the last of these barriers)
+            if constexpr (PERSIST) {
+                if (j == n_tiles - 1 && tl == 0) lds_claim = claim;
+            }
             __syncthreads();
         }
-        pv_mfma(1, (n_tiles - 1) & 3, 1);      // keys 32..63 of the last tile
-#pragma unroll
-        for (int qt = 0; qt < 2; ++qt)
-#pragma unroll
-            for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) o_acc[qt][dt][e] *= o_pending[qt];
     }
 
     // ---- Probabilities are stored in the 16-bit type relative to a reference point that follows the scores lazily.
@@ -601,6 +722,28 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
     bool again = false;
 #pragma unroll
     for (int w = 0; w < NW; ++w) again = again || lds_ref[w] != 0.f;
+    bool has_after = false;
+    if constexpr (PERSIST) {
+        if (has_next) {
+            const uint32_t t2 = 2u * per_cls + static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(lds_claim)));
+            has_after = t2 < n_items;
+            if (has_after) decode_item(t2, aa_seq_start, aa_L, aa_head, aa_q0);
+        }
+        // Q of the next item: requested now, needed behind this item's epilogue (a block that is computed again
+        // still needs its own Q; the next item then starts cold)
+        if (!again && has_next) load_q(tl, nx_seq_start, nx_L, nx_head, nx_q0);
+    }
+    if (!idle) {
+        if (!again) {
+            pv_mfma(1, (ring + n_tiles - 1) & 3, 1);      // keys 32..63 of the last tile
+#pragma unroll
+            for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o_acc[qt][dt][e] *= o_pending[qt];
+        }
+    }
     if (again) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // no direct load is in flight any more
         m_base = 0.f;                                           // the seeds are absolute now
@@ -658,16 +801,16 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
         for (int qt = 0; qt < 2; ++qt) m_run[qt] = m_row[qt] == -INFINITY ? 0.f : m_row[qt];
         __syncthreads();                                        // the epilogue reuses the stages
     }
-    if (idle) return;
 
     // ---- epilogue of a split workgroup: unnormalised outputs, reference point and row sum of its key share
-    if (piece != nullptr) {
+    const int wave_e = tl >> 6, r_e = tl & 31, h_e = (tl >> 5) & 1;
+    if (!idle && piece != nullptr) {
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) {
             const float l_tot = sum_across_halves(l_run[qt]);
-            const int local_row = (wave * 2 + qt) * 32 + r;
+            const int local_row = (wave_e * 2 + qt) * 32 + r_e;
             if (q0 + local_row < L) {
-                float *op = piece + local_row * kHeadDim + 4 * h;
+                float *op = piece + local_row * kHeadDim + 4 * h_e;
 #pragma unroll
                 for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
@@ -675,33 +818,33 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
                         *reinterpret_cast<f32x4 *>(op + 32 * dt + 8 * g) =
                             f32x4{o_acc[qt][dt][4 * g], o_acc[qt][dt][4 * g + 1], o_acc[qt][dt][4 * g + 2],
                                   o_acc[qt][dt][4 * g + 3]};
-                if (h == 0) {
+                if (h_e == 0) {
                     piece[kBlockM * kHeadDim + local_row] = m_run[qt];
                     piece[kBlockM * (kHeadDim + 1) + local_row] = l_tot;
                 }
             }
         }
-        return;
     }
 
     // ---- epilogue: normalise, write O (and LSE).  In the accumulators a lane holds 8-byte pieces of one output row,
     // 32 rows per store instruction; written like that, a wavefront's 32 stores touch 32 rows each and queue up in the
-    // memory pipeline for microseconds (2.5 of the 30 us of a workgroup on an 800-token segment).  Each wavefront
-    // therefore passes its two 32 x 64 tiles through 4 KiB of LDS (16-byte chunk c of row r at chunk c ^ (r & 7)) and
-    // stores whole 128-byte rows, eight rows per instruction.  The LDS comes from stages that nothing reads or fills
-    // any more: K of the last tile and of the two tiles staged behind it (landed before the loop's last barrier; only
-    // the stage after those is still being filled) and V of the tile before the last.
-    {
-        const int last = n_tiles - 1;
+    // memory pipeline for microseconds.  Each wavefront therefore passes its two 32 x 64 tiles through 4 KiB of LDS
+    // (16-byte chunk c of row r at chunk c ^ (r & 7)) and stores whole 128-byte rows, eight rows per instruction.
+    // The LDS comes from stages nothing reads or fills any more: K of the item's last tile and V of the one before
+    // (their next loads are issued behind at least one barrier from here), for wavefronts 4 .. 7 the K stages of the
+    // two tiles staged ahead of the end, which have landed.
+    if (!idle && piece == nullptr) {
+        const int last = ring + n_tiles - 1;
         uint16_t *slot_base = wave_u < 2   ? &lds_k[last & 3][2048 * wave_u]
-                              : wave_u < 4 ? &lds_v[(last + 3) & 3][2048 * (wave_u - 2)]
+                              : wave_u < 4 ? &lds_v[(last - 1) & 3][2048 * (wave_u - 2)]
                               : wave_u < 6 ? &lds_k[(last + 1) & 3][2048 * (wave_u - 4)]
                                            : &lds_k[(last + 2) & 3][2048 * (wave_u - 6)];
+        const int lane_e = tl & 63;
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) {
             const float l_tot = sum_across_halves(l_run[qt]);
             const float inv = 1.0f / l_tot;
-            const int row = q0 + (wave * 2 + qt) * 32 + r;
+            const int row = q0 + (wave_e * 2 + qt) * 32 + r_e;
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
@@ -709,17 +852,17 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
                     u32x2 w;
                     w[0] = E::pack2(o_acc[qt][dt][4 * g] * inv, o_acc[qt][dt][4 * g + 1] * inv);
                     w[1] = E::pack2(o_acc[qt][dt][4 * g + 2] * inv, o_acc[qt][dt][4 * g + 3] * inv);
-                    *reinterpret_cast<u32x2 *>(slot_base + r * 64 + (((4 * dt + g) ^ (r & 7)) << 3) + 4 * h) = w;
+                    *reinterpret_cast<u32x2 *>(slot_base + r_e * 64 + (((4 * dt + g) ^ (r_e & 7)) << 3) + 4 * h_e) = w;
                 }
-            if (row < L && h == 0 && a.lse)
+            if (row < L && h_e == 0 && a.lse)
                 a.lse[static_cast<int64_t>(head) * a.total + seq_start + row] =
                     (m_run[qt] + __log2f(l_tot)) * 0.6931471805599453f;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int tr = 8 * i + (lane >> 3);                        // row of the tile, 8 lanes per row
-                const int c = (lane & 7) ^ (tr & 7);                       // the chunk this lane finds at position lane % 8
-                const u32x4 v = *reinterpret_cast<const u32x4 *>(slot_base + tr * 64 + ((lane & 7) << 3));
-                const int orow = q0 + (wave * 2 + qt) * 32 + tr;
+                const int tr = 8 * i + (lane_e >> 3);                      // row of the tile, 8 lanes per row
+                const int c = (lane_e & 7) ^ (tr & 7);                     // the chunk this lane finds at position lane % 8
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(slot_base + tr * 64 + ((lane_e & 7) << 3));
+                const int orow = q0 + (wave_e * 2 + qt) * 32 + tr;
                 if (orow < L) {
                     uint16_t *op = a.out + static_cast<int64_t>(seq_start + orow) * a.o_rs + head * a.o_hs + 8 * c;
                     if (a.out_wide) {
@@ -731,6 +874,63 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_pipe_kernel(const AttnArgs a
                 }
             }
         }
+    }
+    if constexpr (!PERSIST) {
+        return;
+    } else {
+        if (!has_next) return;
+        ring = (ring + n_tiles) & 3;
+        cold = again;
+        seq_start = nx_seq_start;
+        L = nx_L;
+        head = nx_head;
+        q0 = nx_q0;
+        k_seg = nx_k_seg;
+        v_seg = nx_v_seg;
+        b_seg = nx_b_seg;
+        b_mis = nx_b_mis;
+        has_next = has_after;
+        nx_seq_start = aa_seq_start;
+        nx_L = aa_L;
+        nx_head = aa_head;
+        nx_q0 = aa_q0;
+    }
+    }   // item loop
+}
+
+// Work queue of a launch of resident workgroups (PERSIST above), built from the segment offsets on the device: one
+// wavefront per class c writes list c - for every (segment, head) unit u = c mod 8 in turn the entries (u << 8 | b) of
+// its query blocks b = 0 .. ceil(L / 256) - 1, full blocks first - together with the length of the list, and clears
+// the class's claim counter.  No empty entries: a bound on the segment lengths that is far above them (a caller that
+// does not want to read the longest segment back) costs nothing.  One launch of one workgroup in front of the
+// attention kernel; 64 units per step and wavefront.
+__global__ __launch_bounds__(512) void attn_items_kernel(const AttnArgs a) {
+    const uint32_t lane = threadIdx.x & 63u, cls = threadIdx.x >> 6;
+    uint32_t *list = a.queue + 16 + static_cast<size_t>(cls) * a.queue_cap;
+    const uint32_t n_units = static_cast<uint32_t>(a.n_units);
+    const uint32_t per_class = n_units > cls ? (n_units - cls + 7u) / 8u : 0u;       // units cls, cls + 8, ...
+    uint32_t carry = 0;
+    for (uint32_t i0 = 0; i0 < per_class; i0 += 64u) {
+        const uint32_t i = i0 + lane, unit = cls + 8u * i;
+        uint32_t nb = 0;
+        if (i < per_class) {
+            int start, len;
+            segment_of(a, static_cast<int>(unit / static_cast<uint32_t>(a.n_heads)), start, len);
+            nb = static_cast<uint32_t>(min((len + 255) / 256, a.n_mblocks));         // (never beyond the list)
+        }
+        uint32_t incl = nb;
+#pragma unroll
+        for (uint32_t d = 1; d < 64u; d <<= 1) {
+            const uint32_t up = __shfl_up(incl, d);
+            if (lane >= d) incl += up;
+        }
+        const uint32_t at = carry + incl - nb;
+        for (uint32_t b = 0; b < nb; ++b) list[at + b] = (unit << 8) | b;
+        carry += __shfl(incl, 63);
+    }
+    if (lane == 0) {
+        a.queue[8 + cls] = carry;
+        a.queue[cls] = 0;
     }
 }
 
@@ -793,9 +993,14 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const AttnArgs a, int
 //    fills its last round; otherwise two 256-query workgroups share a CU and the last round finishes early.
 //  - With a work buffer the query blocks of that last round are cut along the keys into `splits` workgroups
 //    each, which fill the chip with short pieces instead; a small kernel combines the pieces.
+//  - Segments of at most kPersistMaxSeqlen keys: with a work buffer the launch is two resident workgroups per CU
+//    that take their query blocks from a queue in the buffer (attn_items_kernel builds it first); without one,
+//    one workgroup per query block as for everything else.
 struct Plan {
     bool wide = false;
     int nb_tail = 0, splits = 1;
+    bool persist = false;
+    int64_t queue_cap = 0;
     int64_t work_bytes = 0;
 };
 
@@ -810,11 +1015,26 @@ int cu_count() {
     return n_cu;
 }
 
-Plan make_plan(int64_t n_seq, int64_t total, int64_t n_heads, int64_t max_seqlen, bool may_split) {
+// Bytes of the work queue of a launch of resident workgroups (0: the shape is not eligible).
+int64_t queue_cap_of(int64_t n_seq, int64_t n_heads, int64_t max_seqlen) {
+    const int64_t units = n_seq * n_heads;
+    if (max_seqlen <= 0 || max_seqlen > kPersistMaxSeqlen || units <= 0 || units > 65536) return 0;
+    return ceil_div(units, 8) * ceil_div(max_seqlen, 256);
+}
+
+Plan make_plan(int64_t n_seq, int64_t total, int64_t n_heads, int64_t max_seqlen, bool may_split, bool work_queue) {
     Plan p;
+    const int64_t units = n_seq * n_heads;
+    if (max_seqlen <= kPersistMaxSeqlen) {
+        if (work_queue && may_split && queue_cap_of(n_seq, n_heads, max_seqlen) > 0) {
+            p.persist = true;
+            p.queue_cap = ceil_div(units, 8) * ceil_div(max_seqlen, 256);
+            p.work_bytes = static_cast<int64_t>(sizeof(uint32_t)) * (16 + 8 * p.queue_cap);
+        }
+        return p;
+    }
     if (max_seqlen < 4096) return p;
     const int n_cu = cu_count();
-    const int64_t units = n_seq * n_heads;
     // one segment: exact; several: half a block of padding per segment on average
     const int64_t expected = n_seq == 1 ? n_heads * ceil_div(total, 512) : n_heads * ceil_div(total + n_seq * 256, 512);
     const int64_t rounds = ceil_div(expected, n_cu);
@@ -851,9 +1071,14 @@ Plan make_plan(int64_t n_seq, int64_t total, int64_t n_heads, int64_t max_seqlen
 
 using namespace come;
 
+extern "C" int64_t come_attn_queue_bytes(int64_t n_seq, int64_t n_heads, int64_t max_seqlen) {
+    const int64_t cap = queue_cap_of(n_seq, n_heads, max_seqlen);
+    return cap > 0 ? static_cast<int64_t>(sizeof(uint32_t)) * (16 + 8 * cap) : 0;
+}
+
 extern "C" int64_t come_attn_work_bytes(int64_t n_seq, int64_t total, int64_t n_heads, int64_t max_seqlen) {
     if (n_seq <= 0 || total <= 0 || n_heads <= 0 || max_seqlen <= 0) return 0;
-    return make_plan(n_seq, total, n_heads, max_seqlen, true).work_bytes;
+    return make_plan(n_seq, total, n_heads, max_seqlen, true, false).work_bytes;
 }
 
 // Address of this device's copy of `scratch` (nullptr + error message on failure).  The array's name is only a
@@ -891,7 +1116,7 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
                                 int64_t o_row_stride, int64_t o_head_stride, float *lse, void *work,
                                 int64_t work_bytes, bool static_work, int flags, void *stream) {
     clear_error();
-    COME_REQUIRE((flags & ~COME_ATTN_FOLD_SCALE) == 0, COME_ERR_INVALID,
+    COME_REQUIRE((flags & ~(COME_ATTN_FOLD_SCALE | COME_ATTN_WORK_QUEUE)) == 0, COME_ERR_INVALID,
                  "come_attn_varlen_fwd: unknown bits in flags (%d)", flags);
     COME_REQUIRE(dtype == COME_BF16 || dtype == COME_F16, COME_ERR_UNSUPPORTED,
                  "come_attn_varlen_fwd: only fp16 and bf16 are supported");
@@ -943,8 +1168,9 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
         a.splits = 1;
         return launch_attn_hd(a, dtype, static_cast<int>(head_dim), max_seqlen, static_cast<hipStream_t>(stream));
     }
-    Plan plan = make_plan(n_seq, total, n_heads, max_seqlen, work != nullptr || static_work);
-    if (static_work && plan.splits > 1) {
+    const bool want_queue = (flags & COME_ATTN_WORK_QUEUE) != 0;
+    Plan plan = make_plan(n_seq, total, n_heads, max_seqlen, work != nullptr || static_work, want_queue);
+    if (static_work && (plan.splits > 1 || plan.persist)) {
         COME_REQUIRE(plan.work_bytes <= kStaticWorkBytes, COME_ERR_UNSUPPORTED,
                      "come_attn_varlen_fwd_static: this launch needs a work buffer of %lld bytes, the built-in one "
                      "holds %lld; use come_attn_varlen_fwd_ws with a buffer of come_attn_work_bytes() bytes",
@@ -953,8 +1179,8 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
         if (work == nullptr) return COME_ERR_HIP;
         work_bytes = kStaticWorkBytes;
     }
-    if (plan.splits > 1 && (work_bytes < plan.work_bytes || (reinterpret_cast<uintptr_t>(work) & 15) != 0))
-        plan = make_plan(n_seq, total, n_heads, max_seqlen, false);        // buffer too small or misaligned: no split
+    if ((plan.splits > 1 || plan.persist) && (work_bytes < plan.work_bytes || (reinterpret_cast<uintptr_t>(work) & 15) != 0))
+        plan = make_plan(n_seq, total, n_heads, max_seqlen, false, false);  // buffer too small or misaligned: neither split nor queue
     const bool wide = plan.wide;
     const int kBlockM = wide ? 512 : 256;
     AttnArgs a{};
@@ -979,6 +1205,8 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
     a.nb_tail = plan.nb_tail;
     a.splits = plan.splits;
     a.work = static_cast<float *>(work);
+    a.queue = static_cast<uint32_t *>(work);
+    a.queue_cap = static_cast<int>(plan.queue_cap);
     a.n_full_wg = ceil_div(n_seq * n_heads, 8) * 8 * a.n_mblocks;
     const int64_t n_wg = a.n_full_wg + ceil_div(n_seq * n_heads, 8) * 8 * (plan.splits > 1 ? plan.nb_tail * plan.splits : 0);
     const int64_t n_cwg = n_seq * n_heads * plan.nb_tail * (kBlockM / 16);       // combine kernel: 16 rows each
@@ -987,18 +1215,35 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
     const dim3 grid(static_cast<unsigned>(n_wg)), block(wide ? 512 : 256);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool exact = (flags & COME_ATTN_FOLD_SCALE) == 0;
-#define COME_ATTN_LAUNCH(DT_, NW_)                                                                              \
-    do {                                                                                                        \
-        if (exact) hipLaunchKernelGGL((attn_fwd_pipe_kernel<DT_, NW_, true>), grid, block, 0, s, a);            \
-        else hipLaunchKernelGGL((attn_fwd_pipe_kernel<DT_, NW_, false>), grid, block, 0, s, a);                 \
+    // short segments with a buffer for the queue: two workgroups per CU that take their items from it
+    const bool persist = plan.persist;
+    if (persist) {
+        hipLaunchKernelGGL(attn_items_kernel, dim3(1), dim3(512), 0, s, a);
+        COME_CHECK_LAUNCH("come_attn_varlen_fwd (work queue)");
+    }
+    const int64_t resident = (2 * static_cast<int64_t>(cu_count())) & ~7ll;
+    const dim3 pgrid(static_cast<unsigned>(n_wg < resident ? n_wg : resident));
+#define COME_ATTN_LAUNCH(DT_, NW_)                                                                                 \
+    do {                                                                                                           \
+        if (exact) hipLaunchKernelGGL((attn_fwd_pipe_kernel<DT_, NW_, true, false>), grid, block, 0, s, a);        \
+        else hipLaunchKernelGGL((attn_fwd_pipe_kernel<DT_, NW_, false, false>), grid, block, 0, s, a);             \
     } while (0)
-    if (wide) {
+#define COME_ATTN_LAUNCH_ITEMS(DT_)                                                                                \
+    do {                                                                                                           \
+        if (exact) hipLaunchKernelGGL((attn_fwd_pipe_kernel<DT_, 4, true, true>), pgrid, block, 0, s, a);          \
+        else hipLaunchKernelGGL((attn_fwd_pipe_kernel<DT_, 4, false, true>), pgrid, block, 0, s, a);               \
+    } while (0)
+    if (persist) {
+        if (dtype == COME_BF16) COME_ATTN_LAUNCH_ITEMS(COME_BF16);
+        else COME_ATTN_LAUNCH_ITEMS(COME_F16);
+    } else if (wide) {
         if (dtype == COME_BF16) COME_ATTN_LAUNCH(COME_BF16, 8);
         else COME_ATTN_LAUNCH(COME_F16, 8);
     } else {
         if (dtype == COME_BF16) COME_ATTN_LAUNCH(COME_BF16, 4);
         else COME_ATTN_LAUNCH(COME_F16, 4);
     }
+#undef COME_ATTN_LAUNCH_ITEMS
 #undef COME_ATTN_LAUNCH
     COME_CHECK_LAUNCH("come_attn_varlen_fwd");
     if (plan.splits > 1) {

@@ -53,7 +53,7 @@ def _pad_head(t: torch.Tensor, head_size: int) -> torch.Tensor:
 
 
 def _forward(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale, causal, window_size, softcap,
-             alibi_slopes, return_softmax, scale_mode="auto"):
+             alibi_slopes, return_softmax, scale_mode="auto", work_queue=False):
     """Shared forward of the plain and the biased operator (``perkey_bias`` may be None)."""
     if softmax_scale is None:
         softmax_scale = qkv.shape[-1] ** (-0.5)
@@ -68,10 +68,11 @@ def _forward(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale,
     tail = (max_seqlen, max_seqlen, dropout_p, softmax_scale, False, causal, int(window_size[0]),
             int(window_size[1]), softcap, return_softmax and dropout_p > 0, None)
     if perkey_bias is None:
-        out_padded, softmax_lse, s_dmask, rng_state = _C.varlen_fwd(*args, *tail, fold_scale=fold)
+        out_padded, softmax_lse, s_dmask, rng_state = _C.varlen_fwd(*args, *tail, fold_scale=fold,
+                                                                    work_queue=work_queue)
     else:
         out_padded, softmax_lse, s_dmask, rng_state = _C.varlen_fwd_w_perkey_bias(*args, perkey_bias, *tail,
-                                                                                  fold_scale=fold)
+                                                                                  fold_scale=fold, work_queue=work_queue)
     out = out_padded if out_padded.shape[-1] == head_size_og else out_padded[..., :head_size_og]
     return out, softmax_lse, s_dmask, rng_state
 
@@ -82,11 +83,12 @@ class _VarlenQKVPacked(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale, causal, window_size,
-                softcap, alibi_slopes, deterministic, return_softmax, is_grad_enabled, op_name, scale_mode):
+                softcap, alibi_slopes, deterministic, return_softmax, is_grad_enabled, op_name, scale_mode,
+                work_queue):
         ctx.op_name = op_name
         out, softmax_lse, s_dmask, rng_state = _forward(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p,
                                                         softmax_scale, causal, window_size, softcap, alibi_slopes,
-                                                        return_softmax, scale_mode)
+                                                        return_softmax, scale_mode, work_queue)
         ctx.mark_non_differentiable(softmax_lse, s_dmask, rng_state)
         return out if not return_softmax else (out, softmax_lse, s_dmask)
 
@@ -96,38 +98,41 @@ class _VarlenQKVPacked(torch.autograd.Function):
 
 
 def _call(op_name, qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale, causal, window_size, softcap,
-          alibi_slopes, deterministic, return_attn_probs, scale_mode):
+          alibi_slopes, deterministic, return_attn_probs, scale_mode, work_queue=False):
     needs_graph = torch.is_grad_enabled() and (qkv.requires_grad
                                                or (perkey_bias is not None and perkey_bias.requires_grad))
     if needs_graph:
         return _VarlenQKVPacked.apply(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale, causal,
                                       window_size, softcap, alibi_slopes, deterministic, return_attn_probs, True,
-                                      op_name, scale_mode)
+                                      op_name, scale_mode, work_queue)
     # inference: nothing to record, skip the autograd.Function machinery (about 10 us of host time per call)
     out, softmax_lse, s_dmask, _ = _forward(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale,
-                                            causal, window_size, softcap, alibi_slopes, return_attn_probs, scale_mode)
+                                            causal, window_size, softcap, alibi_slopes, return_attn_probs, scale_mode,
+                                            work_queue)
     return out if not return_attn_probs else (out, softmax_lse, s_dmask)
 
 
 def flash_attn_varlen_qkvpacked_func(qkv, cu_seqlens, max_seqlen, dropout_p=0.0, softmax_scale=None, causal=False,
                                      window_size=(-1, -1), softcap=0.0, alibi_slopes=None, deterministic=False,
-                                     return_attn_probs=False, *, scale_mode="auto"):
+                                     return_attn_probs=False, *, scale_mode="auto", work_queue=False):
     """``qkv [total, 3, nheads, headdim]``, ``cu_seqlens [batch + 1] int32`` -> ``out [total, nheads, headdim]``
     (plus ``softmax_lse [nheads, total]`` and an empty tensor when ``return_attn_probs``).
 
     ``scale_mode`` (keyword only, not in the reference): ``"exact"`` applies ``softmax_scale`` in fp32 to every score,
     ``"folded"`` folds it into a 16-bit q, ``"auto"`` (default) folds only for a ``qkv`` that carries a small enough
-    ``come_qk_bound`` (see ``FOLD_SCALE_MAX_LOGIT``)."""
+    ``come_qk_bound`` (see ``FOLD_SCALE_MAX_LOGIT``).  ``work_queue`` (keyword only): segments of at most 2048 keys are
+    computed by resident workgroups that take their query blocks from a work list built on the device; same bits,
+    measured slower than the default grid on every shape tried (kept for segment mixes that defeat a static grid)."""
     return _call("flash_attn_varlen_qkvpacked_func", qkv, cu_seqlens, max_seqlen, None, dropout_p, softmax_scale,
-                 causal, window_size, softcap, alibi_slopes, deterministic, return_attn_probs, scale_mode)
+                 causal, window_size, softcap, alibi_slopes, deterministic, return_attn_probs, scale_mode, work_queue)
 
 
 def flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p=0.0,
                                                    softmax_scale=None, causal=False, window_size=(-1, -1),
                                                    softcap=0.0, alibi_slopes=None, deterministic=False,
-                                                   return_attn_probs=False, *, scale_mode="auto"):
+                                                   return_attn_probs=False, *, scale_mode="auto", work_queue=False):
     """Same as :func:`flash_attn_varlen_qkvpacked_func` with ``softmax(Q K^T * scale + perkey_bias[key]) V``;
     ``perkey_bias [total]`` has the dtype of ``qkv`` and is indexed like the packed keys."""
     return _call("flash_attn_varlen_qkvpacked_func_w_perkey_bias", qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p,
                  softmax_scale, causal, window_size, softcap, alibi_slopes, deterministic, return_attn_probs,
-                 scale_mode)
+                 scale_mode, work_queue)

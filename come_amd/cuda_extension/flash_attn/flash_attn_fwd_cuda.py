@@ -54,7 +54,8 @@ def _placeholders(dev: torch.device, dtype: torch.dtype):
 
 def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
                      perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal,
-                     window_size_left, window_size_right, softcap, return_softmax, gen, fold_scale=False):
+                     window_size_left, window_size_right, softcap, return_softmax, gen, fold_scale=False,
+                     work_queue=False):
     _check(q.dtype in (torch.float16, torch.bfloat16), "FlashAttention only support fp16 and bf16 data type")
     _check(k.dtype == q.dtype, "query and key must have the same dtype")
     _check(v.dtype == q.dtype, "query and value must have the same dtype")
@@ -123,7 +124,7 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
         padded = _varlen_fwd_impl(*(torch.nn.functional.pad(t, [0, kernel_width - head_size]) for t in (q, k, v)),
                                   None, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
                                   perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, False, is_causal,
-                                  window_size_left, window_size_right, softcap, return_softmax, gen, fold_scale)
+                                  window_size_left, window_size_right, softcap, return_softmax, gen, fold_scale, work_queue)
         narrow = padded[0][..., :head_size]
         if out_ is not None:
             _check(out_.dtype == q.dtype and tuple(out_.shape) == (total_q, num_heads, head_size),
@@ -155,6 +156,10 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
             # work buffer for the key-split tail of long launches (0 bytes: the launch does not use one)
             work_bytes = (lib.come_attn_work_bytes(batch_size, total_q, num_heads, max_seqlen_k)
                           if head_size == 64 else 0)
+            flags = _lib.COME_ATTN_FOLD_SCALE if fold_scale else 0
+            if work_queue and head_size == 64:
+                work_bytes = max(work_bytes, lib.come_attn_queue_bytes(batch_size, num_heads, max_seqlen_k))
+                flags |= _lib.COME_ATTN_WORK_QUEUE
             work = torch.empty(work_bytes, dtype=torch.uint8, device=dev) if work_bytes > 0 else None
             _lib.check(lib.come_attn_varlen_fwd_ws(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.dtype_code(q.dtype),
@@ -162,8 +167,7 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
                 cu_seqlens_q.data_ptr(), batch_size, total_q, num_heads, head_size,
                 _lib.ptr(perkey_bias), max_seqlen_k, float(softmax_scale),
                 out.data_ptr(), out.stride(0), out.stride(1), softmax_lse.data_ptr(),
-                _lib.ptr(work), work_bytes, _lib.COME_ATTN_FOLD_SCALE if fold_scale else 0,
-                _lib.current_stream(dev)))
+                _lib.ptr(work), work_bytes, flags, _lib.current_stream(dev)))
         else:
             out.zero_()
             softmax_lse.fill_(math.inf)
@@ -172,24 +176,26 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
 
 def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
                max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal,
-               window_size_left, window_size_right, softcap, return_softmax, gen=None, *, fold_scale=False):
+               window_size_left, window_size_right, softcap, return_softmax, gen=None, *, fold_scale=False,
+               work_queue=False):
     """Forward pass (variable length).  Returns ``[out, softmax_lse, p, rng_state]``.
 
-    ``fold_scale`` (keyword only, not in the reference): fold ``softmax_scale`` into a 16-bit q instead of applying
-    it in fp32 to every score (``COME_ATTN_FOLD_SCALE`` of the C ABI); for callers that know their logits stay within
-    about +-10 nats."""
+    Keyword only, not in the reference: ``fold_scale`` folds ``softmax_scale`` into a 16-bit q instead of applying
+    it in fp32 to every score (``COME_ATTN_FOLD_SCALE`` of the C ABI), for callers that know their logits stay within
+    about +-10 nats; ``work_queue`` runs short segments as resident workgroups fed from a device-side work list
+    (``COME_ATTN_WORK_QUEUE``: same bits, slower on every shape measured, see the header)."""
     return _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table,
                             alibi_slopes, None, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                             zero_tensors, is_causal, window_size_left, window_size_right, softcap,
-                            return_softmax, gen, fold_scale)
+                            return_softmax, gen, fold_scale, work_queue)
 
 
 def varlen_fwd_w_perkey_bias(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table,
                              alibi_slopes, perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                              zero_tensors, is_causal, window_size_left, window_size_right, softcap,
-                             return_softmax, gen=None, *, fold_scale=False):
-    """Forward pass (variable length) with a per-key additive bias (``fold_scale``: see :func:`varlen_fwd`)."""
+                             return_softmax, gen=None, *, fold_scale=False, work_queue=False):
+    """Forward pass (variable length) with a per-key additive bias (keywords: see :func:`varlen_fwd`)."""
     return _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table,
                             alibi_slopes, perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                             zero_tensors, is_causal, window_size_left, window_size_right, softcap,
-                            return_softmax, gen, fold_scale)
+                            return_softmax, gen, fold_scale, work_queue)

@@ -49,8 +49,18 @@ typedef enum come_dtype {
  *                          2^-9 of its size: inside 1e-2 max-abs / 1e-3 mean-abs for logits within about +-10 nats
  *                          (q / k LayerNorm with gains near 1), outside it from about +-20 nats on.  A caller that
  *                          knows such a bound for its logits may set it; nothing else should.
+ *   COME_ATTN_WORK_QUEUE   (come_attn_varlen_fwd_ws / _static, segments of at most 2048 keys, at most 65 536
+ *                          (segment, head) units) the launch is two resident workgroups per CU which take their
+ *                          256-query blocks from a queue in the work buffer - a one-workgroup kernel builds it from
+ *                          cu_seqlens first: lists of (unit, block) items without empty entries - and stage the
+ *                          first tiles of their next item during the last iterations of the current one.  Needs
+ *                          come_attn_queue_bytes(...) bytes of buffer; without them the flag is ignored.  Same bits
+ *                          as the default launch (one workgroup per query block).  Measured 5 - 12 % SLOWER than the
+ *                          default on every shape tried: the hardware's own dispatch staggers and re-ages the two
+ *                          workgroups of a CU, which a resident pair cannot.  Kept for callers whose segment mix
+ *                          defeats a static grid (max_seqlen far above most lengths costs nothing here).
  */
-enum { COME_ATTN_FOLD_SCALE = 1 };
+enum { COME_ATTN_FOLD_SCALE = 1, COME_ATTN_WORK_QUEUE = 2 };
 
 /* Library version (major * 10000 + minor * 100 + patch). */
 int come_version(void);
@@ -252,6 +262,9 @@ int come_attn_varlen_fwd(const void *q, const void *k, const void *v, int dtype,
  * src/cuda_extension/flash_attn/src/flash_fwd_launch_template.h:99-157, unreachable from the varlen forward).
  */
 int64_t come_attn_work_bytes(int64_t n_seq, int64_t total, int64_t n_heads, int64_t max_seqlen);
+/* Buffer size for COME_ATTN_WORK_QUEUE (0: that shape never uses a queue).  No counterpart in the reference, whose
+ * grid is (ceil(max_seqlen / 128), batch, heads) (src/cuda_extension/flash_attn/src/flash_fwd_launch_template.h:63-64). */
+int64_t come_attn_queue_bytes(int64_t n_seq, int64_t n_heads, int64_t max_seqlen);
 int come_attn_varlen_fwd_ws(const void *q, const void *k, const void *v, int dtype,
                             int64_t q_row_stride, int64_t q_head_stride,
                             int64_t k_row_stride, int64_t k_head_stride,

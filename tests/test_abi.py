@@ -110,7 +110,7 @@ def test_every_entry_point_rejects_bad_arguments_on_the_host():
     rejected(lib.come_attn_varlen_fwd(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 64,
                                       None, 10, 0.125, None, 64, 64, None, 0, None), "NULL")
     rejected(lib.come_attn_varlen_fwd(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 64,
-                                      None, 10, 0.125, None, 64, 64, None, 6, None), "flags")
+                                      None, 10, 0.125, None, 64, 64, None, 12, None), "flags")
     rejected(lib.come_attn_varlen_fwd_ws(None, None, None, BF16, 64, 64, 64, 64, 64, 64, None, 1, 10, 1, 48,
                                          None, 10, 0.125, None, 64, 64, None, None, 0, 0, None), "head_dim")
     rejected(lib.come_qk_norm_rope(None, None, F32, 64, 64, 64, 64, 4, 1, 64, 1, None, None, None, None, 1e-5,
