@@ -76,6 +76,10 @@ def load() -> ctypes.CDLL:
                     "(run `python -m come_amd.build`). There is no fallback implementation."
                 )
             lib = ctypes.CDLL(LIB_PATH)
+            lib.come_version.restype = ctypes.c_int
+            if lib.come_version() < 200:
+                raise RuntimeError(f"{LIB_PATH} is an older build of libcome_hip (version {lib.come_version()}): its "
+                                   "attention entry points take no `flags` argument; rebuild with `python -m come_amd.build`")
             for name, (restype, argtypes) in SIGNATURES.items():
                 fn = getattr(lib, name)
                 fn.restype = restype

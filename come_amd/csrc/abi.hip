@@ -21,6 +21,7 @@ void clear_error() { g_last_error.clear(); }
 
 }  // namespace come
 
-extern "C" int come_version(void) { return 100; }
+// 0.2.0: the attention entry points take a `flags` argument (the process-wide scale switch is gone)
+extern "C" int come_version(void) { return 200; }
 
 extern "C" const char *come_last_error(void) { return come::g_last_error.c_str(); }

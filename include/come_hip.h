@@ -62,7 +62,7 @@ typedef enum come_dtype {
  */
 enum { COME_ATTN_FOLD_SCALE = 1, COME_ATTN_WORK_QUEUE = 2 };
 
-/* Library version (major * 10000 + minor * 100 + patch). */
+/* Library version (major * 10000 + minor * 100 + patch); 200 = 0.2.0, the first with `flags` on the attention entry points. */
 int come_version(void);
 
 /* Message of the last failing call made by this thread ("" if none). */

@@ -95,7 +95,7 @@ def test_scale_mode_choice_follows_the_bound_attached_by_the_prologue():
     assert _norm_bound(None, None, 64, torch.float16) == pytest.approx(8.0)
     # the bound really bounds the norm of any normalised head
     x = torch.randn(1000, 64) * 5 + 3
-    y = torch.nn.functional.layer_norm(x, (64,), ln.weight, ln.bias)
+    y = torch.nn.functional.layer_norm(x, (64,), ln.weight.detach(), ln.bias.detach())
     assert float(y.norm(dim=-1).max()) <= _norm_bound(ln.weight, ln.bias, 64, torch.float32)
 
     t = torch.zeros(4, 3, 2, 64)
