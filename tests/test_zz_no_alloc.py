@@ -93,3 +93,52 @@ def test_static_matches_workspace_entry_twice_then_rejects_oversize():
     assert "come_attn_varlen_fwd_static" in msg and "come_attn_varlen_fwd_ws" in msg and str(limit) in msg
     torch.cuda.synchronize()
     assert torch.isnan(out.float()).all()                         # untouched
+
+
+def test_static_entry_point_inside_a_captured_graph():
+    """The caller the entry point exists for: the launch is recorded into a HIP graph (the address of the built-in
+    array is looked up before the capture through ``come_attn_static_work_bytes``) and replayed several times, with
+    eager work and synchronisations of the program between the replays; every replay reproduces the eager result bit
+    for bit, on changed inputs as well."""
+    lib = _lib.load()
+    assert lib.come_attn_static_work_bytes() == 64 << 20          # also resolves the array's address on this device
+    lengths = [12288]                                             # uses the key-split tail, i.e. the array
+    assert lib.come_attn_work_bytes(1, 12288, HEADS, 12288) > 0
+    qkv, bias, cu = _inputs(lengths, 7)
+    total = sum(lengths)
+    out = torch.empty(total, HEADS, D, dtype=qkv.dtype, device=DEV)
+    lse = torch.empty(HEADS, total, dtype=torch.float32, device=DEV)
+    st, want, want_lse = _call("static", qkv, bias, cu, max(lengths))
+    assert st == 0
+    torch.cuda.synchronize()
+
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        st, _, _ = _call("static", qkv, bias, cu, max(lengths), out=out, lse=lse)      # warm-up on the capturing stream
+        assert st == 0
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            st, _, _ = _call("static", qkv, bias, cu, max(lengths), out=out, lse=lse)
+        assert st == 0, lib.come_last_error()
+    torch.cuda.current_stream().wait_stream(side)
+    for replay in range(3):
+        out.fill_(float("nan"))
+        lse.fill_(float("nan"))
+        scratch_work = torch.randn(1 << 20, device=DEV).sum()      # the program's own eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want) and torch.equal(lse, want_lse), f"replay {replay}"
+        assert bool(torch.isfinite(scratch_work))
+    # new inputs in the same buffers: the graph holds pointers, not data
+    qkv2, bias2, _ = _inputs(lengths, 8)
+    st, want2, want2_lse = _call("static", qkv2, bias2, cu, max(lengths))
+    torch.cuda.synchronize()
+    qkv.copy_(qkv2)
+    bias.copy_(bias2)
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, want2) and torch.equal(lse, want2_lse)
