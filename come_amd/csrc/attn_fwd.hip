@@ -23,8 +23,8 @@
 //   (The reference adds bias / scale to the raw scores, flash_fwd_kernel.h:30-55, and
 //   subtracts the scaled running maximum inside exp2, softmax.h:76-88.)  Keys beyond the end of
 //   the segment get scores of -inf and probabilities of exactly 0.
-//   The reference point of a row moves lazily (only when a half-tile's row sum leaves the range the
-//   16-bit probabilities keep their precision in).  A workgroup in which a stored probability left
+//   The reference point of a row moves lazily (only when its row sum - bf16: the running one, fp16: that of a
+//   half-tile - leaves the range the 16-bit probabilities keep their precision in).  A workgroup in which a stored probability left
 //   the 16-bit range altogether raises a flag on the loop's last barrier and then computes its
 //   query block again, tile by tile, with a running maximum per row: any finite scores are exact.
 //   That is the instantiation COME_ATTN_FOLD_SCALE selects.  The default one (EXACT) keeps Q as it is: the
@@ -92,10 +92,12 @@ __device__ inline bool locate_block(const AttnArgs &a, int &mblk, int &head, int
 //   S'' = (c q) . k + bias log2(e) - m,      c = softmax_scale log2(e)
 // Q is multiplied by c once (and rounded back to 16 bit); bias log2(e) - m is the initial value of the
 // accumulator (one subtraction per score on the vector ALU).  m is the row maximum of the first 32 keys and
-// is moved, by a power of two, only when a half-tile's row sum leaves a safe range (sums and outputs are
+// is moved, by a power of two, only when the row sum leaves a safe range (sums and outputs are
 // then rescaled as in the usual online softmax); softmax is invariant to the choice of m, and fp32 / 16-bit
-// floats keep full relative precision for probabilities above 1.  The steady state therefore spends one
-// subtraction, one exp2, half a pack and half a dot per score on the vector ALU and nothing else.
+// floats keep full relative precision for probabilities above 1.  Row sums are taken on the matrix pipe too
+// (the rounded probabilities times a matrix of ones, v_mfma_f32_16x16x32), so the steady state spends one
+// exp2 and half a pack per score on the vector ALU (plus one multiplication where the scale is applied in fp32)
+// and six additions per half-tile for the range check.
 // -------------------------------------------------------------------------------------
 constexpr int kStages = 4;
 // Launches whose segments are at most this long walk their work items in resident workgroups (PERSIST below): a few
@@ -104,10 +106,11 @@ constexpr int64_t kPersistMaxSeqlen = 2048;
 
 // Range of the probabilities relative to the reference point of their row.  They are stored in the 16-bit type of
 // the inputs: bf16 has the exponent range of fp32, fp16 reaches only 65504 and loses precision below 2^-14.
-//   kSumLimit  a half-tile row sum above this moves the reference point of the row up
+//   kSumLimit  a row sum above this (bf16: the running sum, fp16: the sum over a half-tile) moves the reference point
+//              of the row up
 //   kMaxGap    a row whose own maximum lies further below the workgroup's reference point keeps its own offset
 template <int DT> struct Range;
-//   kHardLimit a half-tile row sum above this may come from probabilities that left the 16-bit type's range
+//   kHardLimit a row sum above this may come from probabilities that left the 16-bit type's range
 //              (infinite, or saturated): the workgroup then computes its block again with a running maximum
 template <> struct Range<COME_BF16> {
     static constexpr float kSumLimit = 1099511627776.f;   // 2^40
@@ -383,7 +386,35 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     float m_run[2] = {0.f, 0.f};  // reference point of the row, log2 units: m_base + delta
     float delta[2] = {0.f, 0.f};  // what the row's reference point differs from m_base by (0 for nearly all rows)
     bool has_delta = false;       // wave-uniform: some row of this wavefront has delta != 0
-    float l_run[2] = {0.f, 0.f};  // per-lane partial row sum
+    float l_run[2] = {0.f, 0.f};  // per-lane partial row sum (outside the key loop: the block that is computed again, the epilogues)
+    // Row sums in the key loop come from the matrix pipe: with the probabilities of a 16-key step as the A operand of
+    // v_mfma_f32_16x16x32 (row m = lane % 16, eight keys per lane: lane group g = lane / 16 holds query m + 16 (g & 1),
+    // keys 8 (g >> 1) ..) and a B operand whose lane group g is all ones in column g & 1 and zero elsewhere, the result
+    // column n = 0 / 1 holds the sums of queries m / m + 16 over the step's 16 keys, whatever order the unit gives the
+    // keys inside a lane.  In the 16 x 16 result a lane holds column lane % 16, rows 4 (lane / 16) .. + 3: the sums of
+    // queries 0 .. 15 sit in lanes 0, 16, 32, 48, those of queries 16 .. 31 in lanes 1, 17, 33, 49, four per lane, and
+    // every other lane holds zeros.  Four such MFMAs per slot (64 cycles of the matrix pipe) replace 16 v_dot2c_f32,
+    // which hold the matrix pipe for as long as eight of them and the vector ALU on top.
+    // bf16 (kChain): the MFMAs accumulate straight onto the running sums and the range check looks at those - a running
+    // sum beyond 2^40 moves the reference point just as well as a half-tile sum beyond it.  fp16: its limit (2^5) is
+    // about the size of the current probabilities, which a running sum says nothing about, so the sums of a slot are
+    // formed on their own and added afterwards.
+    constexpr bool kChain = DT == COME_BF16;
+    f32x4 l_acc[2];               // running row sums in that layout
+    const u32x4 ones_sel = ((lane & 15) == ((lane >> 4) & 1))
+                               ? u32x4{E::kOne | (E::kOne << 16), E::kOne | (E::kOne << 16), E::kOne | (E::kOne << 16), E::kOne | (E::kOne << 16)}
+                               : zero4();
+    const int sum_lane = (r >> 4) + 16 * ((r & 15) >> 2);         // where this lane's query keeps its row sum (element r & 3)
+    // row sum of this lane's query out of that layout (a few LDS permutes: rare path and loop exit only)
+    auto row_value = [&](const f32x4 &v) __attribute__((always_inline)) -> float {
+        float out = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float t = __shfl(v[j], sum_lane);
+            out = (r & 3) == j ? t : out;
+        }
+        return out;
+    };
 
     // scores of both query tiles against half-tile `half` of the K tile in `buf`, into buffer b: the accumulators
     // start from the LDS bias values of their keys and collect the four k-steps of (c Q) K^T
@@ -426,8 +457,8 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     // previous slot).  Every MFMA is followed by a chunk of vector work and fragments are requested two
     // fragments (four MFMAs) ahead, so an in-order wavefront always has independent work behind each
     // MFMA.  sched_barrier keeps the compiler from regrouping the chunks.
-    // Returns through sum[qt] the row sums of this lane over the half-tile.
-    auto slot = [&](int X, int Y, int kbuf, int khalf, int vbuf, int vhalf, float (&sum)[2]) __attribute__((always_inline)) {
+    // Returns through ssum[qt] the row sums of the half-tile (layout of l_acc).
+    auto slot = [&](int X, int Y, int kbuf, int khalf, int vbuf, int vhalf, f32x4 (&ssum)[2]) __attribute__((always_inline)) {
         // fragments 0..3: V (u, dt) of the P V MFMAs 0..7; fragments 4..7: K k-steps of the score MFMAs 8..15.
         // P V goes first: the probabilities of buffer Y die while those of buffer X are born, and the score
         // registers of buffer Y are not needed before half of buffer X has been consumed.
@@ -458,8 +489,9 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
         };
         request(0);
         request(1);
-        sum[0] = 0.f;
-        sum[1] = 0.f;
+        const f32x4 zero4f = {0.f, 0.f, 0.f, 0.f};
+        f32x4 &dst0 = kChain ? l_acc[0] : ssum[0];
+        f32x4 &dst1 = kChain ? l_acc[1] : ssum[1];
         float p0 = 0.f, p1 = 0.f;
 #pragma unroll
         for (int c = 0; c < 16; ++c) {
@@ -475,7 +507,10 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
                 const int pc = c - 1, qt = pc >> 3, w = pc & 7;
                 const uint32_t pw = E::pack2_prob(p0, p1);
                 p_frag[X][qt][w >> 2][w & 3] = pw;
-                sum[qt] = E::dot2_ones(pw, sum[qt]);
+                // a 16-key step of a query tile is complete: its row sums
+                if (pc == 3) dst0 = E::mfma16(p_frag[X][0][0], ones_sel, kChain ? l_acc[0] : zero4f);
+                if (pc == 7) dst0 = E::mfma16(p_frag[X][0][1], ones_sel, dst0);
+                if (pc == 11) dst1 = E::mfma16(p_frag[X][1][0], ones_sel, kChain ? l_acc[1] : zero4f);
             }
             float s0 = s_acc[X][c >> 3][2 * (c & 7)], s1 = s_acc[X][c >> 3][2 * (c & 7) + 1];
             if (EXACT) {
@@ -490,11 +525,11 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
         {
             const uint32_t pw = E::pack2_prob(p0, p1);
             p_frag[X][1][1][3] = pw;
-            sum[1] = E::dot2_ones(pw, sum[1]);
+            dst1 = E::mfma16(p_frag[X][1][1], ones_sel, dst1);
         }
         // the decision that follows the slot is tied to its end, so that the branch cannot be moved
         // above the probability chunks
-        asm volatile("" : "+v"(sum[1]) : "v"(p_frag[X][1][1][3]));
+        asm volatile("" : "+v"(dst1) : "v"(p_frag[X][1][1][3]));
     };
 
     // O[qt] *= f, in place.  Written as asm so that the accumulator tuples keep their registers across a
@@ -520,8 +555,14 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     float o_pending[2] = {1.f, 1.f};
     bool any_pending = false;                  // wave-uniform
     bool overflowed = false;                   // wave-uniform: some half-tile row sum exceeded kHardLimit
-    auto finish_slot = [&](int Y, const float (&sum)[2]) __attribute__((always_inline)) {
-        const bool bad = !(sum[0] <= kSumLimit) || !(sum[1] <= kSumLimit);
+    auto finish_slot = [&](int Y, const f32x4 (&ssum)[2]) __attribute__((always_inline)) {
+        // sums are not negative: if the four rows of a lane together stay within the limit, each of them does
+        // (written so that a NaN counts as beyond it)
+        const f32x4 &c0 = kChain ? l_acc[0] : ssum[0];
+        const f32x4 &c1 = kChain ? l_acc[1] : ssum[1];
+        const float t0 = (c0[0] + c0[1]) + (c0[2] + c0[3]);
+        const float t1 = (c1[0] + c1[1]) + (c1[2] + c1[3]);
+        const bool bad = !(t0 <= kSumLimit) || !(t1 <= kSumLimit);
         if (__any(bad) || any_pending || has_delta) {
             // the asm arithmetic below reads MFMA results; the compiler cannot see that, so the wait states an
             // MFMA result needs before a vector instruction may read it are spent here explicitly
@@ -530,11 +571,11 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
             for (int qt = 0; qt < 2; ++qt) {
                 if (any_pending) scale_o(qt, o_pending[qt]);
-                float row_sum = sum[qt];
+                // of this lane's query: over all 32 keys of the half-tile, or (kChain) over all keys so far
+                float row_sum = row_value(kChain ? l_acc[qt] : ssum[qt]);
                 asm volatile("" : "+v"(row_sum));       // keeps the arithmetic of this rare path inside the branch
                 overflowed = overflowed || __any(!(row_sum <= Range<DT>::kHardLimit));
-                int shift = row_sum <= kSumLimit ? 0 : max(__builtin_amdgcn_frexp_expf(row_sum) - 2, 1);
-                shift = static_cast<int>(max_across_halves(static_cast<float>(shift)));   // both half-waves of a row agree
+                const int shift = row_sum <= kSumLimit ? 0 : max(__builtin_amdgcn_frexp_expf(row_sum) - 2, 1);
                 const float down = __builtin_amdgcn_exp2f(static_cast<float>(-shift));
                 delta[qt] += static_cast<float>(shift);
                 m_run[qt] += static_cast<float>(shift);
@@ -545,15 +586,21 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
                     asm volatile("v_sub_f32 %0, %0, %1" : "+v"(t) : "v"(d));
                     s_acc[Y][qt][e] = t;
                 }
-                l_run[qt] = (l_run[qt] + row_sum) * down;
+                // the running sums, where they live: element j of a lane belongs to query 16 (lane % 16) + 4 (lane / 16) + j
+                // (lanes whose column is neither 0 nor 1 hold zeros and stay zero)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float dj = __shfl(down, (16 * (lane & 15) + 4 * (lane >> 4) + j) & 31);
+                    l_acc[qt][j] = (kChain ? l_acc[qt][j] : l_acc[qt][j] + ssum[qt][j]) * dj;
+                }
                 o_pending[qt] = down;
                 again = again || __any(shift != 0);
             }
             any_pending = again;
             has_delta = __any(delta[0] != 0.f || delta[1] != 0.f);
-        } else {
-            l_run[0] += sum[0];
-            l_run[1] += sum[1];
+        } else if (!kChain) {
+            l_acc[0] += ssum[0];
+            l_acc[1] += ssum[1];
         }
     };
 
@@ -598,6 +645,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
         o_acc[qt][0] = zero16;
         o_acc[qt][1] = zero16;
         l_run[qt] = 0.f;
+        l_acc[qt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
             p_frag[b][qt][0] = zero4();
@@ -695,7 +743,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
             load_bias(j + 4, kb);      // raw bias runs one more tile ahead (converted between the slots of iteration j+2)
             stage_k(j + 3, kb3);       // K(j+3) replaces K(j-1), V(j+2) replaces V(j-2): both idle since the
             stage_v(j + 2, kb2);       // last barrier; they are first read two barriers from now
-            float sum[2];
+            f32x4 sum[2];
             peek_bias(kb2);
             // slot a: keys 0..31 of tile j become probabilities; scores of keys 32..63; P V of keys 32..63 of tile j-1
             slot(0, 1, kb, 1, kb3, 1, sum);
@@ -735,6 +783,12 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     }
     if (!idle) {
         if (!again) {
+            // the row sums leave the layout of the key loop: the lower half-wave carries the total, the upper one nothing
+#pragma unroll
+            for (int qt = 0; qt < 2; ++qt) {
+                const float total = row_value(l_acc[qt]);
+                l_run[qt] = h == 0 ? total : 0.f;
+            }
             pv_mfma(1, (ring + n_tiles - 1) & 3, 1);      // keys 32..63 of the last tile
 #pragma unroll
             for (int qt = 0; qt < 2; ++qt)

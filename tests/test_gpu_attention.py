@@ -294,7 +294,7 @@ def test_key_beyond_the_range_inside_a_key_split_piece():
         torch.testing.assert_close(lse[:, row], torch.logsumexp(scores, -1), atol=2e-2, rtol=1e-3)
 
 
-@pytest.mark.parametrize("kind", ["ramp", "jump", "late_rows", "descending"])
+@pytest.mark.parametrize("kind", ["ramp", "jump", "late_rows", "descending", "plateau"])
 def test_reference_point_moves(kind):
     """Scores that grow by many orders of magnitude along the keys: the kernel keeps probabilities relative
     to a per-row reference point taken from the first keys and has to move it (rare path) without losing
@@ -309,6 +309,11 @@ def test_reference_point_moves(kind):
     elif kind == "late_rows":
         bias = torch.zeros(L)
         qkv[:, 1, :, :] *= torch.linspace(0.2, 6.0, L)[:, None, None].bfloat16()     # later keys score far higher
+    elif kind == "plateau":
+        # 22 nats up from key 200 on and staying there: no 32 keys add up to 2^40 times the first keys' sum, but the
+        # running row sum passes it some 300 keys later, and again never after the reference point has moved
+        bias = torch.zeros(L)
+        bias[200:] = 22.0
     else:
         bias = torch.linspace(40.0, -40.0, L)
     bias = bias.bfloat16()
