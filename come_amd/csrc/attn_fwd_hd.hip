@@ -141,7 +141,16 @@ __global__ __launch_bounds__(256) void attn_fwd_hd_kernel(const AttnArgs a) {
 #pragma unroll
     for (int dt = 0; dt < kDTiles; ++dt) o_acc[dt] = zero16;
     float m_ref = -INFINITY;      // reference point of the row, log2 units
-    float l_run = 0.f;            // per-lane partial row sum
+    // Row sums come from the matrix pipe: the probabilities of a 16-key step as the A operand of v_mfma_f32_16x16x32
+    // (row m = lane % 16; lane group g = lane / 16 holds query m + 16 (g & 1)) against a B operand whose lane group g
+    // is all ones in column g & 1: result column 0 / 1 holds the sums of queries m / m + 16.  A lane of the result
+    // holds column lane % 16, rows 4 (lane / 16) .. + 3, so the running sums of queries 0 .. 15 sit in lanes 0, 16, 32,
+    // 48 and those of queries 16 .. 31 in lanes 1, 17, 33, 49, four per lane; all other lanes hold zeros.
+    f32x4 l_acc = {0.f, 0.f, 0.f, 0.f};
+    const u32x4 ones_sel = ((lane & 15) == ((lane >> 4) & 1))
+                               ? u32x4{E::kOne | (E::kOne << 16), E::kOne | (E::kOne << 16), E::kOne | (E::kOne << 16), E::kOne | (E::kOne << 16)}
+                               : u32x4{0u, 0u, 0u, 0u};
+    const int owner_base = (16 * (lane & 15) + 4 * (lane >> 4)) & 31;     // element j of l_acc belongs to query owner_base + j
 
     // k-step ks of the scores of half-tile `half` of the K tile in `buf`
     auto score_step = [&](f32x16 &s, int buf, int half, int ks) __attribute__((always_inline)) {
@@ -180,10 +189,10 @@ __global__ __launch_bounds__(256) void attn_fwd_hd_kernel(const AttnArgs a) {
         if (moved) {
             down = move ? __builtin_amdgcn_exp2f(m_ref - mx) : 1.f;
             m_ref = move ? mx : m_ref;
-            l_run *= down;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) l_acc[j] *= __shfl(down, owner_base + j);
         }
         const float ref = m_ref == -INFINITY ? 0.f : m_ref;     // a row that has seen masked keys only
-        float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < 8; ++w) {
             if (kKSteps >= 8) {
@@ -195,9 +204,9 @@ __global__ __launch_bounds__(256) void attn_fwd_hd_kernel(const AttnArgs a) {
             const uint32_t pw = E::pack2_prob(__builtin_amdgcn_exp2f(x[2 * w] - ref),
                                               __builtin_amdgcn_exp2f(x[2 * w + 1] - ref));
             p[w >> 2][w & 3] = pw;
-            sum = E::dot2_ones(pw, sum);
+            if (w == 3) l_acc = E::mfma16(p[0], ones_sel, l_acc);
         }
-        l_run += sum;
+        l_acc = E::mfma16(p[1], ones_sel, l_acc);
         if (moved) {
 #pragma unroll
             for (int dt = 0; dt < kDTiles; ++dt)
@@ -240,7 +249,15 @@ __global__ __launch_bounds__(256) void attn_fwd_hd_kernel(const AttnArgs a) {
     if (idle) return;
 
     // ---- epilogue: normalise, write O (and LSE)
-    const float l_tot = sum_across_halves(l_run);
+    float l_tot = 0.f;
+    {
+        const int sum_lane = (r >> 4) + 16 * ((r & 15) >> 2);          // where this lane's query keeps its sum (element r & 3)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float t = __shfl(l_acc[j], sum_lane);
+            l_tot = (r & 3) == j ? t : l_tot;
+        }
+    }
     const float inv = 1.0f / l_tot;
     const int row = q0 + wave * 32 + r;
     if (row < L) {
