@@ -508,7 +508,8 @@ def bench_bias_overhead(device):
 def bench_qk_prologue(device, rows=(25536, 43968), iters=200, warmup=20):
     """q / k LayerNorm + 2-D RoPE in place on the packed ``qkv [P, 3, 16, 64]`` bf16 (one launch through the C ABI),
     over 4 rotating tensors (each launch touches 2/3 of 157 MB at P = 25 536).  Algorithmic bytes: q and k read and
-    written once."""
+    written once.  ``k_only``: the same launch with a null q (half the bytes), what remains of the pass when the q half
+    is left to the attention kernel (``defer_q``)."""
     import torch
     from come_amd import _lib
     from come_amd.common import RotaryPositionEmbedding2D
@@ -524,10 +525,10 @@ def bench_qk_prologue(device, rows=(25536, 43968), iters=200, warmup=20):
         pos = torch.randint(0, 38, (P, 2), device=device)
         state = {"i": 0}
 
-        def step():
+        def step(k_only=False):
             i = state["i"] = (state["i"] + 1) % 4
             q, k = sets[i][:, 0], sets[i][:, 1]
-            _lib.check(lib.come_qk_norm_rope(q.data_ptr(), k.data_ptr(), _lib.COME_BF16, q.stride(0), q.stride(1),
+            _lib.check(lib.come_qk_norm_rope(None if k_only else q.data_ptr(), k.data_ptr(), _lib.COME_BF16, q.stride(0), q.stride(1),
                                              k.stride(0), k.stride(1), P, H, 64, 1, params[0].data_ptr(),
                                              params[1].data_ptr(), params[2].data_ptr(), params[3].data_ptr(), 1e-5,
                                              pos.data_ptr(), cos_t.data_ptr(), sin_t.data_ptr(), 38, stream))
@@ -535,8 +536,12 @@ def bench_qk_prologue(device, rows=(25536, 43968), iters=200, warmup=20):
         _, ms = time_loop(step, iters, warmup)
         nbytes = P * 2 * H * 64 * 2 * 2
         gbs = nbytes / (ms / iters * 1e-3) / 1e9
+        _, ms_k = time_loop(lambda: step(True), iters, warmup)
+        gbs_k = nbytes / 2 / (ms_k / iters * 1e-3) / 1e9
         out["P=%d" % P] = {"us_per_call": round(ms / iters * 1e3, 2), "algorithmic_bytes": nbytes, "GBs": round(gbs, 1),
-                           "frac": round(gbs / PEAK_HBM_GBS, 4)}
+                           "frac": round(gbs / PEAK_HBM_GBS, 4),
+                           "k_only": {"us_per_call": round(ms_k / iters * 1e3, 2), "algorithmic_bytes": nbytes // 2,
+                                      "GBs": round(gbs_k, 1), "frac": round(gbs_k / PEAK_HBM_GBS, 4)}}
         del sets
         torch.cuda.empty_cache()
     return out
@@ -626,6 +631,44 @@ def bench_scale_mode(device, mode, steps=10, warmup=3):
                          "kernel": "attn_fwd_pipe_kernel<bf16, 8, %s>" % ("true" if mode == "exact" else "false")}}
 
 
+def bench_deferred_q_prologue(device, steps=20, warmup=5):
+    """The headline workload with the q half of the prologue (LayerNorm + 2-D rotary embedding) done by the attention
+    kernel on the query fragments it loads (``prepare_packed_self_attention_qkv(..., defer_q=True)``), next to the
+    two-step path on the same tensors: per layer call, full in-place pass + attention against k-only pass + attention
+    with the prologue.  fp32 scale on every score in both."""
+    import torch
+    from come_amd.common import RotaryPositionEmbedding2D, prepare_packed_self_attention_qkv
+    from come_amd.cuda_extension import flash_attn_varlen_qkvpacked_func_w_perkey_bias
+
+    w = make_attention_workload(device)
+    P, max_len = w["qkv"].shape[0], max(w["lens"])
+    norms = [torch.nn.LayerNorm(64, eps=1e-6).to(device=device, dtype=torch.bfloat16) for _ in range(2)]
+    rope = RotaryPositionEmbedding2D(100.0)
+    pos = torch.randint(0, 38, (P, 2), device=device)
+    res = {}
+    for name, defer in (("two_step", False), ("deferred_q", True)):
+        # the pass rewrites q / k in place: every step works on a LayerNorm'd tensor again, which is what it would see
+        qkv = w["qkv"].clone()
+
+        def prologue():
+            return prepare_packed_self_attention_qkv(qkv, norms[0], norms[1], rope, pos, torch.bfloat16, max_position=37,
+                                                     defer_q=defer)
+
+        def attention():
+            return flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv, w["cu"], max_len, perkey_bias=w["bias"],
+                                                                  softmax_scale=0.125, scale_mode="exact")
+
+        with torch.no_grad():
+            prologue()
+            _, ms_p = time_loop(prologue, 10 * steps, 10 * warmup)
+            _, ms_a = time_loop(attention, steps, warmup)
+        res[name] = {"prologue_us": round(ms_p / (10 * steps) * 1e3, 1), "attention_ms": round(ms_a / steps, 4),
+                     "sum_ms": round(ms_p / (10 * steps) + ms_a / steps, 4)}
+    res["saved_us_per_layer_call"] = round((res["two_step"]["sum_ms"] - res["deferred_q"]["sum_ms"]) * 1e3, 1)
+    res["workload"] = "headline attention workload (P = 47384 packed rows, 16 heads x 64), q / k LayerNorm + 2-D RoPE"
+    return res
+
+
 def bench_other_widths(device, steps=20, warmup=40):
     """The biased varlen attention at the head dimensions beside 64 that have their own kernel instance (32 and 128):
     one segment of 16 384 tokens, 16 heads, bf16, bias log(count) on 30 % of the keys."""
@@ -672,7 +715,7 @@ def bench_e2e(device, frames=32, depth=24, reps=5, height=518, width=518, ratio=
     ``within_tolerance`` says whether the merged model stayed within the stated relative L1 of the unmerged one on
     the pixels of unmerged windows; the same check is an assertion in tests/test_gpu_e2e_full.py."""
     import torch
-    from come_amd.harness import AggregatorConfig, AlternatingAggregator, relative_l1
+    from come_amd.harness import AggregatorConfig, AlternatingAggregator, deferred_q_prologue, relative_l1
     from come_amd.token_merger import CoMe_2D_TokenMerger
 
     torch.manual_seed(0)
@@ -682,19 +725,21 @@ def bench_e2e(device, frames=32, depth=24, reps=5, height=518, width=518, ratio=
     merger = CoMe_2D_TokenMerger(cfg.specials, 3, 3, ratio, allow_remainder=True)
     gh, gw = height // 14, width // 14
 
-    def timed(m):
-        out = model(images, merger=m)                           # warm-up (allocator, GEMM heuristics)
+    def timed(m, prologue=None):
+        out = model(images, merger=m, prologue=prologue)        # warm-up (allocator, GEMM heuristics)
         torch.cuda.synchronize()
         times = []
         for _ in range(reps):
             t0 = time.perf_counter()
-            out = model(images, merger=m)
+            out = model(images, merger=m, prologue=prologue)
             torch.cuda.synchronize()
             times.append((time.perf_counter() - t0) * 1e3)
         return out, sorted(times)[len(times) // 2]
 
     dense, dense_ms = timed(None)
     merged, merged_ms = timed(merger)
+    # the same forward with the q half of every attention prologue left to the attention kernel: the same bits
+    fused, fused_ms = timed(merger, deferred_q_prologue)
     mh, mw = gh // 3, gw // 3
     mask = merged["merge_mask"].reshape(frames, mh, mw)
     keep = torch.ones(frames, gh, gw, dtype=torch.bool, device=device)
@@ -706,6 +751,8 @@ def bench_e2e(device, frames=32, depth=24, reps=5, height=518, width=518, ratio=
                         f"3x3 merge from block {cfg.merge_block} at r={ratio} ({merged['tokens_packed']} packed tokens)",
             "merged_ms": round(merged_ms, 2), "unmerged_ms": round(dense_ms, 2),
             "speedup": round(dense_ms / merged_ms, 3), "reps": reps, "statistic": "median wall time per forward",
+            "merged_deferred_q_prologue_ms": round(fused_ms, 2),
+            "deferred_q_prologue_same_bits": bool(torch.equal(fused["maps"], merged["maps"])),
             "rel_l1_unmerged_windows": round(rel, 5), "rel_l1_tolerance": 5e-2, "within_tolerance": bool(rel <= 5e-2),
             "finite": bool(torch.isfinite(merged["maps"]).all())}
 
@@ -821,7 +868,8 @@ def main():
         elif args.only == "widths":
             print(json.dumps({"only": "widths", **bench_other_widths(device, args.steps, args.warmup)}))
         elif args.only == "prologue":
-            print(json.dumps({"only": "prologue", **bench_qk_prologue(device, iters=args.steps, warmup=args.warmup)}))
+            print(json.dumps({"only": "prologue", **bench_qk_prologue(device, iters=args.steps, warmup=args.warmup),
+                              "q_half_in_attention": bench_deferred_q_prologue(device)}))
         elif args.only == "refmerge":
             print(json.dumps({"only": "refmerge", **bench_reference_merge_shapes(device)}))
         elif args.only == "bias":
@@ -888,6 +936,7 @@ def main():
         other["merge_caller_dtypes"] = bench_merge_caller_dtypes(device)
         other["reference_merge_microbench_shapes"] = bench_reference_merge_shapes(device)
         other["qk_prologue"] = bench_qk_prologue(device)
+        other["qk_prologue"]["q_half_in_attention"] = bench_deferred_q_prologue(device)
         other["frame_attention"] = bench_frame_attention(device, w)
         other["bias_overhead"] = bench_bias_overhead(device)
         other["attention_exact_scale"] = bench_scale_mode(device, "exact")

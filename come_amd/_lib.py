@@ -26,6 +26,14 @@ _ptr = ctypes.c_void_p
 _int = ctypes.c_int
 _f32 = ctypes.c_float
 
+
+
+class QPrologue(ctypes.Structure):
+    """``come_q_prologue`` of the header: the q-side arguments of ``come_qk_norm_rope`` for ``come_attn_varlen_fwd_qp``."""
+    _fields_ = [("apply_norm", _int), ("eps", _f32), ("weight", _ptr), ("bias", _ptr), ("positions", _ptr),
+                ("cos_table", _ptr), ("sin_table", _ptr), ("n_pos", _i64)]
+
+
 # name -> (restype, argtypes); must list every function declared in include/come_hip.h
 SIGNATURES = {
     "come_version": (_int, []),
@@ -48,6 +56,9 @@ SIGNATURES = {
     "come_attn_varlen_fwd_ws": (_int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64,
                                        _ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _f32,
                                        _ptr, _i64, _i64, _ptr, _ptr, _i64, _int, _ptr]),
+    "come_attn_varlen_fwd_qp": (_int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64,
+                                       _ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _f32,
+                                       _ptr, _i64, _i64, _ptr, _ptr, _i64, ctypes.POINTER(QPrologue), _int, _ptr]),
     "come_attn_static_work_bytes": (_i64, []),
     "come_attn_varlen_fwd_static": (_int, [_ptr, _ptr, _ptr, _int, _i64, _i64, _i64, _i64, _i64, _i64,
                                            _ptr, _i64, _i64, _i64, _i64, _ptr, _i64, _f32,
@@ -77,9 +88,10 @@ def load() -> ctypes.CDLL:
                 )
             lib = ctypes.CDLL(LIB_PATH)
             lib.come_version.restype = ctypes.c_int
-            if lib.come_version() < 200:
-                raise RuntimeError(f"{LIB_PATH} is an older build of libcome_hip (version {lib.come_version()}): its "
-                                   "attention entry points take no `flags` argument; rebuild with `python -m come_amd.build`")
+            if lib.come_version() < 201:
+                raise RuntimeError(f"{LIB_PATH} is an older build of libcome_hip (version {lib.come_version()}, this "
+                                   "binding needs 0.2.1: `flags` on the attention entry points, "
+                                   "come_attn_varlen_fwd_qp); rebuild with `python -m come_amd.build`")
             for name, (restype, argtypes) in SIGNATURES.items():
                 fn = getattr(lib, name)
                 fn.restype = restype

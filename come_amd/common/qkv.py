@@ -9,6 +9,8 @@ updated in place, as in the reference; there is no out-of-place (autograd) branc
 
 from __future__ import annotations
 
+import dataclasses
+
 import torch
 
 from .. import _lib
@@ -45,6 +47,21 @@ def _norm_params(norm):
     raise RuntimeError(f"q_norm / k_norm must be LayerNorm or Identity, got {type(norm).__name__}")
 
 
+@dataclasses.dataclass
+class DeferredQPrologue:
+    """The q half of the prologue, left to the attention kernel (``come_attn_varlen_fwd_qp``): what
+    ``prepare_packed_self_attention_qkv(..., defer_q=True)`` attaches to the tensor it returns as ``come_q_prologue``.
+    Holds the tensors the kernel reads, so that they live as long as the packed tensor does."""
+    apply_norm: bool
+    eps: float
+    weight: torch.Tensor | None
+    bias: torch.Tensor | None
+    positions: torch.Tensor | None
+    cos_table: torch.Tensor | None
+    sin_table: torch.Tensor | None
+    n_pos: int
+
+
 _BOUND_CACHE: dict = {}
 
 
@@ -64,7 +81,8 @@ def _norm_bound(weight, bias, head_dim: int, run_dtype) -> float:
 
 
 def prepare_packed_self_attention_qkv(qkv: torch.Tensor, q_norm, k_norm, rope, pos: torch.Tensor | None,
-                                      run_dtype: torch.dtype, max_position: int | None = None) -> torch.Tensor:
+                                      run_dtype: torch.dtype, max_position: int | None = None, *,
+                                      defer_q: bool = False) -> torch.Tensor:
     """Normalises the packed q and k (``qkv [P, 3, H, D]``) and applies the 2-D RoPE, in place.
 
     ``rope`` is an object with ``base_frequency`` or ``base`` (or ``None``), ``pos [P, 2]`` / ``[1, P, 2]`` integer
@@ -74,6 +92,12 @@ def prepare_packed_self_attention_qkv(qkv: torch.Tensor, q_norm, k_norm, rope, p
     When q and k are LayerNorm'd, the returned tensor carries ``come_qk_bound``: an upper bound of ``|q . k|`` over
     all pairs, ``(sqrt(D) max|gain_q| + |bias_q|) (sqrt(D) max|gain_k| + |bias_k|)`` (the rotation keeps norms; 2 %
     are added for its rounding).  The attention operators use it to choose how ``softmax_scale`` is applied.
+
+    ``defer_q`` (keyword only, not in the reference; head_dim 64): only k is rewritten here; q stays the raw
+    projection and the returned tensor carries ``come_q_prologue``, from which the attention operators of this
+    package normalise and rotate the query rows as their kernel loads them - the same bits as the in-place pass,
+    without reading and writing q once more.  For callers that hand the tensor straight to the attention operator
+    (as ``bias_attention.py:100-137`` of the reference does) and read q nowhere else.
     """
     if torch.is_grad_enabled() and qkv.requires_grad:
         raise RuntimeError("prepare_packed_self_attention_qkv is forward only (in place); run it under torch.no_grad()")
@@ -116,9 +140,11 @@ def prepare_packed_self_attention_qkv(qkv: torch.Tensor, q_norm, k_norm, rope, p
             rope = _TABLES.setdefault(float(base), RotaryPositionEmbedding2D(float(base)))
         cos_t, sin_t = rope.tables(D, n_pos, dev, run_dtype)
     q, k = qkv[:, 0], qkv[:, 1]
+    if defer_q and D != 64:
+        raise RuntimeError(f"defer_q needs head_dim 64 (the attention kernel that applies the q prologue), got {D}")
     lib = _lib.load()
     with torch.cuda.device(dev):
-        _lib.check(lib.come_qk_norm_rope(q.data_ptr(), k.data_ptr(), _lib.dtype_code(run_dtype),
+        _lib.check(lib.come_qk_norm_rope(None if defer_q else q.data_ptr(), k.data_ptr(), _lib.dtype_code(run_dtype),
                                          q.stride(0), q.stride(1), k.stride(0), k.stride(1), P, H, D,
                                          1 if apply_q else 0, _lib.ptr(qw), _lib.ptr(qb), _lib.ptr(kw), _lib.ptr(kb),
                                          q_eps, _lib.ptr(positions), _lib.ptr(cos_t), _lib.ptr(sin_t), n_pos,
@@ -128,4 +154,8 @@ def prepare_packed_self_attention_qkv(qkv: torch.Tensor, q_norm, k_norm, rope, p
             _norm_bound(k_norm.weight, k_norm.bias, D, run_dtype)
     elif hasattr(qkv, "come_qk_bound"):
         del qkv.come_qk_bound
+    if defer_q and (apply_q or use_rope):
+        qkv.come_q_prologue = DeferredQPrologue(apply_q, q_eps, qw, qb, positions, cos_t, sin_t, n_pos)
+    elif hasattr(qkv, "come_q_prologue"):
+        del qkv.come_q_prologue
     return qkv

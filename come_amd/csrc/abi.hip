@@ -22,6 +22,7 @@ void clear_error() { g_last_error.clear(); }
 }  // namespace come
 
 // 0.2.0: the attention entry points take a `flags` argument (the process-wide scale switch is gone)
-extern "C" int come_version(void) { return 200; }
+// 0.2.1: come_attn_varlen_fwd_qp; come_qk_norm_rope skips a null q or k
+extern "C" int come_version(void) { return 201; }
 
 extern "C" const char *come_last_error(void) { return come::g_last_error.c_str(); }

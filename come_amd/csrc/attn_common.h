@@ -27,6 +27,15 @@ struct AttnArgs {
     // 8 item counts, then 8 lists of queue_cap entries (unit << 8 | query block)
     uint32_t *queue;
     int queue_cap;
+    // optional prologue on the query rows, applied as the kernel loads them: LayerNorm over the head (qp_norm; gain
+    // and shift [64] in the tensor dtype, either may be null) and the 2-D rotary embedding (qp_pos [total, 2] (y, x),
+    // null: none; tables [qp_n_pos, 16] in the tensor dtype).  q in memory is then the raw projection.
+    int qp_on, qp_norm;
+    const void *qp_gamma, *qp_beta;
+    float qp_eps;
+    const int64_t *qp_pos;
+    const void *qp_cos, *qp_sin;
+    int64_t qp_n_pos;
 };
 
 namespace {

@@ -31,6 +31,7 @@
 //   accumulator starts from (b_k - m_q) / c and every score is multiplied by c in fp32 in front of the exponential,
 //   which is the reference's arithmetic (bias / scale added to the raw scores, scale applied inside exp2).
 #include "attn_common.h"
+#include "qk_math.h"
 
 #include <mutex>
 
@@ -245,8 +246,64 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
                                              E::to_f32(static_cast<uint16_t>(raw >> 16)) * a.scale_log2);
                 }
     };
+    // The prologue of the attention (q LayerNorm + 2-D rotary embedding, qkv.py:31-39 of the reference's common
+    // package) on the fragments just loaded, with the arithmetic and the summation order of the stand-alone pass, so
+    // that the fragments hold the bits that pass would have written to memory.  A lane holds chunks 2 ks + h of its
+    // query's head (ks = 0 .. 3): the rotation partner of a chunk (c ^ 2) is in the same lane, the neighbour in the
+    // sums (c ^ 1) in lane l ^ 32.
+    auto prepare_q = [&](int tl, int start, int len, int first) __attribute__((always_inline)) {
+        using C = QkChunk<DT>;
+        using V = Vec16<DT>;
+        const int hh = (tl >> 5) & 1;
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+            uint4 word[4];
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) word[ks] = __builtin_bit_cast(uint4, qf[qt][ks]);
+            if (a.qp_norm) {
+                float part[4];
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) part[ks] = sum_across_halves(C::sum(word[ks]));
+                const float mean = C::mean_of((part[0] + part[1]) + (part[2] + part[3]));
+                float f[4][8];
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    V::unpack(word[ks], f[ks]);
+                    part[ks] = sum_across_halves(C::center(f[ks], mean));
+                }
+                const float rstd = C::inv_std((part[0] + part[1]) + (part[2] + part[3]), a.qp_eps);
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    float g[8], b[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) g[i] = 1.f, b[i] = 0.f;
+                    if (a.qp_gamma != nullptr) V::unpack(static_cast<const uint4 *>(a.qp_gamma)[2 * ks + hh], g);
+                    if (a.qp_beta != nullptr) V::unpack(static_cast<const uint4 *>(a.qp_beta)[2 * ks + hh], b);
+                    word[ks] = C::scale(f[ks], rstd, g, b);
+                }
+            }
+            if (a.qp_pos != nullptr) {
+                const int row = first + ((tl >> 6) * 2 + qt) * 32 + (tl & 31);
+                const int64_t token = start + min(row, len - 1);
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {                 // y: chunks 0 - 3 (ks 0, 1), x: chunks 4 - 7 (ks 2, 3)
+                    const int entry = (C::table_row(a.qp_pos[token * 2 + half], a.qp_n_pos) * 16 + hh * 8) * V::ELEM_BYTES;
+                    float c[8], sn[8], lo[8], hi[8];
+                    V::unpack(*reinterpret_cast<const uint4 *>(static_cast<const char *>(a.qp_cos) + entry), c);
+                    V::unpack(*reinterpret_cast<const uint4 *>(static_cast<const char *>(a.qp_sin) + entry), sn);
+                    V::unpack(word[2 * half], lo);
+                    V::unpack(word[2 * half + 1], hi);
+                    word[2 * half] = C::rotate(lo, hi, c, sn, C::one_and_sign(false));
+                    word[2 * half + 1] = C::rotate(hi, lo, c, sn, C::one_and_sign(true));
+                }
+            }
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) qf[qt][ks] = __builtin_bit_cast(u32x4, word[ks]);
+        }
+    };
     if constexpr (!PERSIST) {
         load_q(tid, seq_start, L, head, q0);
+        if (a.qp_on) prepare_q(tid, seq_start, L, q0);
         scale_q();
     }
     // ---- global -> LDS staging.  Wavefront w fills rows 16 w .. 16 w + 15 of a tile with two direct
@@ -1168,7 +1225,8 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
                                 int64_t n_seq, int64_t total, int64_t n_heads, int64_t head_dim,
                                 const void *perkey_bias, int64_t max_seqlen, float softmax_scale, void *out,
                                 int64_t o_row_stride, int64_t o_head_stride, float *lse, void *work,
-                                int64_t work_bytes, bool static_work, int flags, void *stream) {
+                                int64_t work_bytes, bool static_work, int flags, void *stream,
+                                const come_q_prologue *qp = nullptr) {
     clear_error();
     COME_REQUIRE((flags & ~(COME_ATTN_FOLD_SCALE | COME_ATTN_WORK_QUEUE)) == 0, COME_ERR_INVALID,
                  "come_attn_varlen_fwd: unknown bits in flags (%d)", flags);
@@ -1202,6 +1260,19 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
                      (reinterpret_cast<uintptr_t>(v) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0,
                  COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd: q/k/v must be 16-byte aligned, out 8-byte aligned");
 
+    if (qp != nullptr) {
+        COME_REQUIRE(head_dim == kHeadDim, COME_ERR_UNSUPPORTED, "come_attn_varlen_fwd_qp: head_dim must be 64");
+        COME_REQUIRE((flags & COME_ATTN_WORK_QUEUE) == 0, COME_ERR_UNSUPPORTED,
+                     "come_attn_varlen_fwd_qp: not available together with COME_ATTN_WORK_QUEUE");
+        COME_REQUIRE(qp->eps >= 0.f, COME_ERR_INVALID, "come_attn_varlen_fwd_qp: eps must be >= 0");
+        const void *aligned[] = {qp->weight, qp->bias, qp->cos_table, qp->sin_table};
+        for (const void *p : aligned)
+            COME_REQUIRE((reinterpret_cast<uintptr_t>(p) & 15) == 0, COME_ERR_INVALID,
+                         "come_attn_varlen_fwd_qp: prologue pointers must be 16-byte aligned");
+        if (qp->positions != nullptr)
+            COME_REQUIRE(qp->cos_table != nullptr && qp->sin_table != nullptr && qp->n_pos > 0 && qp->n_pos < (1 << 24),
+                         COME_ERR_INVALID, "come_attn_varlen_fwd_qp: positions need cos / sin tables with 0 < n_pos < 2^24");
+    }
     if (head_dim != kHeadDim) {               // the other widths: one kernel, no work buffer
         AttnArgs a{};
         a.q = static_cast<const uint16_t *>(q);
@@ -1261,6 +1332,17 @@ static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int
     a.work = static_cast<float *>(work);
     a.queue = static_cast<uint32_t *>(work);
     a.queue_cap = static_cast<int>(plan.queue_cap);
+    if (qp != nullptr && (qp->apply_norm || qp->positions != nullptr)) {
+        a.qp_on = 1;
+        a.qp_norm = qp->apply_norm ? 1 : 0;
+        a.qp_gamma = qp->weight;
+        a.qp_beta = qp->bias;
+        a.qp_eps = qp->eps;
+        a.qp_pos = qp->positions;
+        a.qp_cos = qp->cos_table;
+        a.qp_sin = qp->sin_table;
+        a.qp_n_pos = qp->n_pos;
+    }
     a.n_full_wg = ceil_div(n_seq * n_heads, 8) * 8 * a.n_mblocks;
     const int64_t n_wg = a.n_full_wg + ceil_div(n_seq * n_heads, 8) * 8 * (plan.splits > 1 ? plan.nb_tail * plan.splits : 0);
     const int64_t n_cwg = n_seq * n_heads * plan.nb_tail * (kBlockM / 16);       // combine kernel: 16 rows each
@@ -1321,6 +1403,19 @@ extern "C" int come_attn_varlen_fwd_ws(const void *q, const void *k, const void 
                                 v_row_stride, v_head_stride, cu_seqlens, n_seq, total, n_heads, head_dim,
                                 perkey_bias, max_seqlen, softmax_scale, out, o_row_stride, o_head_stride, lse,
                                 work, work_bytes, false, flags, stream);
+}
+
+extern "C" int come_attn_varlen_fwd_qp(const void *q, const void *k, const void *v, int dtype, int64_t q_row_stride,
+                                       int64_t q_head_stride, int64_t k_row_stride, int64_t k_head_stride,
+                                       int64_t v_row_stride, int64_t v_head_stride, const int32_t *cu_seqlens,
+                                       int64_t n_seq, int64_t total, int64_t n_heads, int64_t head_dim,
+                                       const void *perkey_bias, int64_t max_seqlen, float softmax_scale, void *out,
+                                       int64_t o_row_stride, int64_t o_head_stride, float *lse, void *work,
+                                       int64_t work_bytes, const come_q_prologue *prologue, int flags, void *stream) {
+    return attn_varlen_fwd_impl(q, k, v, dtype, q_row_stride, q_head_stride, k_row_stride, k_head_stride,
+                                v_row_stride, v_head_stride, cu_seqlens, n_seq, total, n_heads, head_dim,
+                                perkey_bias, max_seqlen, softmax_scale, out, o_row_stride, o_head_stride, lse,
+                                work, work_bytes, false, flags, stream, prologue);
 }
 
 extern "C" int come_attn_varlen_fwd(const void *q, const void *k, const void *v, int dtype, int64_t q_row_stride,

@@ -15,6 +15,7 @@
 // The pass is bound by its in-place access pattern (4 KiB read and written out of every 6 KiB row of
 // the packed projection), not by arithmetic: loads and stores carry the non-temporal hint.
 #include "come_common.h"
+#include "qk_math.h"
 
 namespace come {
 namespace {
@@ -64,45 +65,18 @@ __device__ inline float group8_sum(float v) {
 
 constexpr int kRowsPerThread = 4;      // consecutive rows per lane: their loads are in flight together
 
-// Packed 16-bit pairs of the storage dtype: sum of a pair, and "first + sign * second", both in fp32 with one
-// rounding (a dot product against packed constants: the products with +-1 are exact).
-template <int DT> struct Pair;
-template <> struct Pair<COME_BF16> {
-    static constexpr uint32_t kOne = 0x3F80u, kMinusOne = 0xBF80u;
-    __device__ static inline float dot(uint32_t w, uint32_t k, float acc) {
-        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(come_bf16x2, w), __builtin_bit_cast(come_bf16x2, k), acc, false);
-    }
-    // the same without an accumulator (written out: the compiler otherwise zeroes a register for the in-place form)
-    __device__ static inline float dot0(uint32_t w, uint32_t k) {
-        float d;
-        asm("v_dot2_f32_bf16 %0, %1, %2, 0" : "=v"(d) : "v"(w), "v"(k));
-        return d;
-    }
-    __device__ static inline uint32_t pack(float lo, float hi) { return pack2_bf16(lo, hi); }
-};
-template <> struct Pair<COME_F16> {
-    static constexpr uint32_t kOne = 0x3C00u, kMinusOne = 0xBC00u;
-    __device__ static inline float dot(uint32_t w, uint32_t k, float acc) {
-        return __builtin_amdgcn_fdot2(__builtin_bit_cast(come_f16x2, w), __builtin_bit_cast(come_f16x2, k), acc, false);
-    }
-    __device__ static inline float dot0(uint32_t w, uint32_t k) {
-        float d;
-        asm("v_dot2_f32_f16 %0, %1, %2, 0" : "=v"(d) : "v"(w), "v"(k));
-        return d;
-    }
-    __device__ static inline uint32_t pack(float lo, float hi) { return pack2_f16(lo, hi); }
-};
-
-// Grid: x = groups of kRowsPerThread tokens, y = 256-thread slices of the 2 (q, k) x n_heads x 8 lanes of a token.
+// Grid: x = groups of kRowsPerThread tokens, y = 256-thread slices of the (q, k) x n_heads x 8 lanes of a token
+// (only the tensors that are given: a null q or k is skipped).
 template <int DT>
 __global__ void __launch_bounds__(256) qk_norm_rope_kernel(const QkArgs a) {
     using V = Vec16<DT>;
-    using W = Pair<DT>;
+    using C = QkChunk<DT>;
     const int j = blockIdx.y * 256 + threadIdx.x;                 // (which, head, lane8) of this lane
     const int per_tensor = a.n_heads * 8;
-    if (j >= 2 * per_tensor) return;                              // the eight lanes of a head leave together
-    const int which = j >= per_tensor ? 1 : 0;
-    const int head = (j - which * per_tensor) >> 3;
+    const int first = a.ptr[0] != nullptr ? 0 : 1, n_tensors = (a.ptr[0] != nullptr ? 1 : 0) + (a.ptr[1] != nullptr ? 1 : 0);
+    if (j >= n_tensors * per_tensor) return;                      // the eight lanes of a head leave together
+    const int which = first + (j >= per_tensor ? 1 : 0);
+    const int head = (j - (which - first) * per_tensor) >> 3;
     const int lane8 = j & 7;
     const int64_t token0 = static_cast<int64_t>(blockIdx.x) * kRowsPerThread;
 
@@ -121,8 +95,7 @@ __global__ void __launch_bounds__(256) qk_norm_rope_kernel(const QkArgs a) {
         if (a.positions != nullptr) {
             // lanes 0-3 hold the y half, lanes 4-7 the x half of a head; lanes {0,1} and {2,3} of a half are
             // rotation partners and read the same 16 angles, 8 each
-            const int64_t pos = a.positions[token * 2 + (lane8 >> 2)];
-            const int pc = pos < 0 ? 0 : (pos >= a.n_pos ? static_cast<int>(a.n_pos) - 1 : static_cast<int>(pos));
+            const int pc = C::table_row(a.positions[token * 2 + (lane8 >> 2)], a.n_pos);
             entry[t] = (pc * 16 + (lane8 & 1) * 8) * V::ELEM_BYTES;
         }
     }
@@ -141,9 +114,8 @@ __global__ void __launch_bounds__(256) qk_norm_rope_kernel(const QkArgs a) {
             for (int i = 0; i < 8; ++i) b[i] = 0.f;
         }
     }
-    constexpr uint32_t kOnes = W::kOne | (W::kOne << 16);
     // the rotated partner enters with sign -1 in the first half of each 32-element block
-    const uint32_t one_and_sign = W::kOne | (((lane8 & 2) ? W::kOne : W::kMinusOne) << 16);
+    const uint32_t one_and_sign = C::one_and_sign((lane8 & 2) != 0);
 
 #pragma unroll
     for (int t = 0; t < kRowsPerThread; ++t) {
@@ -151,34 +123,20 @@ __global__ void __launch_bounds__(256) qk_norm_rope_kernel(const QkArgs a) {
         float f[8];
         if (a.apply_norm) {
             // mean from the packed words, then the usual two passes in registers
-            float s = W::dot0(word.x, kOnes);
-            s = W::dot(word.y, kOnes, s);
-            s = W::dot(word.z, kOnes, s);
-            s = W::dot(word.w, kOnes, s);
-            const float mean = group8_sum(s) * (1.0f / 64.0f);
+            const float mean = C::mean_of(group8_sum(C::sum(word)));
             V::unpack(word, f);
-            float q = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                f[i] -= mean;
-                q = fmaf(f[i], f[i], q);
-            }
-            const float rstd = rsqrtf(group8_sum(q) * (1.0f / 64.0f) + a.eps);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) f[i] = fmaf(f[i] * rstd, g[i], b[i]);
-            word = V::pack(f);                                   // the normalised value is rounded once
+            const float q = C::center(f, mean);
+            const float rstd = C::inv_std(group8_sum(q), a.eps);
+            word = C::scale(f, rstd, g, b);                      // the normalised value is rounded once
         }
         if (a.positions != nullptr) {
             V::unpack(word, f);
-            float c[8], sn[8];
+            float c[8], sn[8], partner[8];
             V::unpack(*reinterpret_cast<const uint4 *>(static_cast<const char *>(a.cos_table) + entry[t]), c);
             V::unpack(*reinterpret_cast<const uint4 *>(static_cast<const char *>(a.sin_table) + entry[t]), sn);
-            // x cos and partner sin are rounded as a pair; their signed sum is one dot product and is rounded by
-            // the final pack
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
-                f[i] = W::dot0(W::pack(f[i] * c[i], lane_move<kSwapQuadHalves>(f[i]) * sn[i]), one_and_sign);
-            word = V::pack(f);
+            for (int i = 0; i < 8; ++i) partner[i] = lane_move<kSwapQuadHalves>(f[i]);
+            word = C::rotate(f, partner, c, sn, one_and_sign);
         }
         if (live[t]) st16_stream(reinterpret_cast<uint4 *>(row + t * row_bytes), word);
     }
@@ -203,12 +161,13 @@ extern "C" int come_qk_norm_rope(void *q, void *k, int dtype,
                  static_cast<long long>(head_dim));
     COME_REQUIRE(total >= 0 && n_heads > 0 && n_heads < (1 << 20), COME_ERR_INVALID, "come_qk_norm_rope: bad sizes");
     if (total == 0) return COME_OK;
-    COME_REQUIRE(q != nullptr && k != nullptr, COME_ERR_INVALID, "come_qk_norm_rope: null q / k");
+    COME_REQUIRE(q != nullptr || k != nullptr, COME_ERR_INVALID, "come_qk_norm_rope: q and k are both null");
     const int64_t strides[4] = {q_row_stride, q_head_stride, k_row_stride, k_head_stride};
-    for (int64_t s : strides)
-        COME_REQUIRE(s >= 64 && s % 8 == 0, COME_ERR_INVALID,
+    for (int i = 0; i < 4; ++i)
+        COME_REQUIRE((i < 2 ? q : k) == nullptr || (strides[i] >= 64 && strides[i] % 8 == 0), COME_ERR_INVALID,
                      "come_qk_norm_rope: strides must be multiples of 8 elements and at least 64");
-    COME_REQUIRE(q_row_stride >= q_head_stride * (n_heads - 1) + 64 && k_row_stride >= k_head_stride * (n_heads - 1) + 64,
+    COME_REQUIRE((q == nullptr || q_row_stride >= q_head_stride * (n_heads - 1) + 64) &&
+                     (k == nullptr || k_row_stride >= k_head_stride * (n_heads - 1) + 64),
                  COME_ERR_INVALID, "come_qk_norm_rope: heads of one row overlap the next row");
     const void *aligned[] = {q, k, q_weight, q_bias, k_weight, k_bias, cos_table, sin_table};
     for (const void *p : aligned)
@@ -235,7 +194,7 @@ extern "C" int come_qk_norm_rope(void *q, void *k, int dtype,
     a.sin_table = sin_table;
     a.n_pos = n_pos;
     const int64_t groups = ceil_div(total, kRowsPerThread);
-    const int64_t slices = ceil_div(2 * n_heads * 8, 256);
+    const int64_t slices = ceil_div(((q != nullptr) + (k != nullptr)) * n_heads * 8, 256);
     COME_REQUIRE(groups < (int64_t{1} << 31) && slices < 65536 && n_pos < (1 << 24), COME_ERR_UNSUPPORTED,
                  "come_qk_norm_rope: too many tokens, heads or positions for one launch");
     const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(slices));

@@ -67,12 +67,12 @@ def _forward(qkv, cu_seqlens, max_seqlen, perkey_bias, dropout_p, softmax_scale,
     args = (q, k, v, None, cu_seqlens, cu_seqlens, None, None, None, alibi_slopes)
     tail = (max_seqlen, max_seqlen, dropout_p, softmax_scale, False, causal, int(window_size[0]),
             int(window_size[1]), softcap, return_softmax and dropout_p > 0, None)
+    # the q half of the prologue, when prepare_packed_self_attention_qkv(..., defer_q=True) left it to the kernel
+    extra = dict(fold_scale=fold, work_queue=work_queue, q_prologue=getattr(qkv, "come_q_prologue", None))
     if perkey_bias is None:
-        out_padded, softmax_lse, s_dmask, rng_state = _C.varlen_fwd(*args, *tail, fold_scale=fold,
-                                                                    work_queue=work_queue)
+        out_padded, softmax_lse, s_dmask, rng_state = _C.varlen_fwd(*args, *tail, **extra)
     else:
-        out_padded, softmax_lse, s_dmask, rng_state = _C.varlen_fwd_w_perkey_bias(*args, perkey_bias, *tail,
-                                                                                  fold_scale=fold, work_queue=work_queue)
+        out_padded, softmax_lse, s_dmask, rng_state = _C.varlen_fwd_w_perkey_bias(*args, perkey_bias, *tail, **extra)
     out = out_padded if out_padded.shape[-1] == head_size_og else out_padded[..., :head_size_og]
     return out, softmax_lse, s_dmask, rng_state
 

@@ -55,7 +55,7 @@ def _placeholders(dev: torch.device, dtype: torch.dtype):
 def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
                      perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal,
                      window_size_left, window_size_right, softcap, return_softmax, gen, fold_scale=False,
-                     work_queue=False):
+                     work_queue=False, q_prologue=None):
     _check(q.dtype in (torch.float16, torch.bfloat16), "FlashAttention only support fp16 and bf16 data type")
     _check(k.dtype == q.dtype, "query and key must have the same dtype")
     _check(v.dtype == q.dtype, "query and value must have the same dtype")
@@ -117,6 +117,8 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
         return t.data_ptr() % 16 == 0 and t.stride(0) % 8 == 0 and t.stride(1) % 8 == 0
 
     kernel_width = 32 if head_size <= 32 else 64 if head_size <= 64 else 128
+    if q_prologue is not None:
+        _check(head_size == 64, "a deferred q prologue needs head_dim 64")
     if head_size != kernel_width:
         # in-between widths run zero-padded on the next kernel width: zero columns change neither q . k nor the
         # other columns of the output (softmax_scale was fixed by the caller from the real width); costs a padded
@@ -124,7 +126,7 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
         padded = _varlen_fwd_impl(*(torch.nn.functional.pad(t, [0, kernel_width - head_size]) for t in (q, k, v)),
                                   None, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
                                   perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, False, is_causal,
-                                  window_size_left, window_size_right, softcap, return_softmax, gen, fold_scale, work_queue)
+                                  window_size_left, window_size_right, softcap, return_softmax, gen, fold_scale, work_queue, q_prologue)
         narrow = padded[0][..., :head_size]
         if out_ is not None:
             _check(out_.dtype == q.dtype and tuple(out_.shape) == (total_q, num_heads, head_size),
@@ -161,13 +163,27 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
                 work_bytes = max(work_bytes, lib.come_attn_queue_bytes(batch_size, num_heads, max_seqlen_k))
                 flags |= _lib.COME_ATTN_WORK_QUEUE
             work = torch.empty(work_bytes, dtype=torch.uint8, device=dev) if work_bytes > 0 else None
-            _lib.check(lib.come_attn_varlen_fwd_ws(
-                q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.dtype_code(q.dtype),
-                q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
-                cu_seqlens_q.data_ptr(), batch_size, total_q, num_heads, head_size,
-                _lib.ptr(perkey_bias), max_seqlen_k, float(softmax_scale),
-                out.data_ptr(), out.stride(0), out.stride(1), softmax_lse.data_ptr(),
-                _lib.ptr(work), work_bytes, flags, _lib.current_stream(dev)))
+            common = (q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.dtype_code(q.dtype),
+                      q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
+                      cu_seqlens_q.data_ptr(), batch_size, total_q, num_heads, head_size,
+                      _lib.ptr(perkey_bias), max_seqlen_k, float(softmax_scale),
+                      out.data_ptr(), out.stride(0), out.stride(1), softmax_lse.data_ptr(),
+                      _lib.ptr(work), work_bytes)
+            if q_prologue is None:
+                _lib.check(lib.come_attn_varlen_fwd_ws(*common, flags, _lib.current_stream(dev)))
+            else:
+                qp = q_prologue
+                for t in (qp.weight, qp.bias, qp.positions, qp.cos_table, qp.sin_table):
+                    _check(t is None or (t.device == dev and t.is_contiguous()),
+                           "the tensors of a deferred q prologue must be contiguous and on the device of q")
+                _check(qp.positions is None or (qp.positions.dtype == torch.int64 and qp.positions.numel() == 2 * total_q),
+                       "the positions of a deferred q prologue must be int64 [total, 2]")
+                for t in (qp.weight, qp.bias, qp.cos_table, qp.sin_table):
+                    _check(t is None or t.dtype == q.dtype, "the tensors of a deferred q prologue must have the dtype of q")
+                desc = _lib.QPrologue(1 if qp.apply_norm else 0, float(qp.eps), _lib.ptr(qp.weight), _lib.ptr(qp.bias),
+                                      _lib.ptr(qp.positions), _lib.ptr(qp.cos_table), _lib.ptr(qp.sin_table),
+                                      int(qp.n_pos))
+                _lib.check(lib.come_attn_varlen_fwd_qp(*common, desc, flags, _lib.current_stream(dev)))
         else:
             out.zero_()
             softmax_lse.fill_(math.inf)
@@ -177,25 +193,27 @@ def _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftp
 def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table, alibi_slopes,
                max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal,
                window_size_left, window_size_right, softcap, return_softmax, gen=None, *, fold_scale=False,
-               work_queue=False):
+               work_queue=False, q_prologue=None):
     """Forward pass (variable length).  Returns ``[out, softmax_lse, p, rng_state]``.
 
     Keyword only, not in the reference: ``fold_scale`` folds ``softmax_scale`` into a 16-bit q instead of applying
     it in fp32 to every score (``COME_ATTN_FOLD_SCALE`` of the C ABI), for callers that know their logits stay within
     about +-10 nats; ``work_queue`` runs short segments as resident workgroups fed from a device-side work list
-    (``COME_ATTN_WORK_QUEUE``: same bits, slower on every shape measured, see the header)."""
+    (``COME_ATTN_WORK_QUEUE``: same bits, slower on every shape measured, see the header); ``q_prologue`` (a
+    ``come_amd.common.qkv.DeferredQPrologue``) makes the kernel normalise and rotate the query rows as it loads them
+    (``come_attn_varlen_fwd_qp``: q is then the raw projection, head_dim 64 only)."""
     return _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table,
                             alibi_slopes, None, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                             zero_tensors, is_causal, window_size_left, window_size_right, softcap,
-                            return_softmax, gen, fold_scale, work_queue)
+                            return_softmax, gen, fold_scale, work_queue, q_prologue)
 
 
 def varlen_fwd_w_perkey_bias(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table,
                              alibi_slopes, perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                              zero_tensors, is_causal, window_size_left, window_size_right, softcap,
-                             return_softmax, gen=None, *, fold_scale=False, work_queue=False):
+                             return_softmax, gen=None, *, fold_scale=False, work_queue=False, q_prologue=None):
     """Forward pass (variable length) with a per-key additive bias (keywords: see :func:`varlen_fwd`)."""
     return _varlen_fwd_impl(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, block_table,
                             alibi_slopes, perkey_bias, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                             zero_tensors, is_causal, window_size_left, window_size_right, softcap,
-                            return_softmax, gen, fold_scale, work_queue)
+                            return_softmax, gen, fold_scale, work_queue, q_prologue)

@@ -68,6 +68,17 @@ def _default_prologue(qkv, q_norm, k_norm, rope_base, pos, max_position):
     return prepare_packed_self_attention_qkv(qkv, q_norm, k_norm, rope, pos, qkv.dtype, max_position=max_position)
 
 
+def deferred_q_prologue(qkv, q_norm, k_norm, rope_base, pos, max_position):
+    """The same prologue with its q half left to the attention kernel (``defer_q=True``): k is rewritten in place, q
+    stays the raw projection and is normalised and rotated as the attention kernel loads it - the same bits, one read
+    and one write of q less per block."""
+    from .common import RotaryPositionEmbedding2D, prepare_packed_self_attention_qkv
+
+    rope = _ROPES.setdefault(rope_base, RotaryPositionEmbedding2D(rope_base))
+    return prepare_packed_self_attention_qkv(qkv, q_norm, k_norm, rope, pos, qkv.dtype, max_position=max_position,
+                                             defer_q=True)
+
+
 _ROPES: dict = {}
 
 

@@ -62,7 +62,7 @@ typedef enum come_dtype {
  */
 enum { COME_ATTN_FOLD_SCALE = 1, COME_ATTN_WORK_QUEUE = 2 };
 
-/* Library version (major * 10000 + minor * 100 + patch); 200 = 0.2.0, the first with `flags` on the attention entry points. */
+/* Library version (major * 10000 + minor * 100 + patch); 200 = 0.2.0, the first with `flags` on the attention entry points; 201 adds come_attn_varlen_fwd_qp. */
 int come_version(void);
 
 /* Message of the last failing call made by this thread ("" if none). */
@@ -311,7 +311,8 @@ int come_attn_varlen_fwd_static(const void *q, const void *k, const void *v, int
  * embedding.
  *
  *   q, k      [total, n_heads, head_dim] views of `dtype` (COME_BF16 or COME_F16), unit stride
- *             inside a head, *_row_stride / *_head_stride in elements; overwritten
+ *             inside a head, *_row_stride / *_head_stride in elements; overwritten.  One of them may be
+ *             NULL: that tensor is skipped (its strides are not looked at)
  *   apply_norm  0 = no normalisation; otherwise y = (x - mean) * rsqrt(var + eps) * weight + bias
  *             over the head_dim elements of a head (biased variance, fp32 arithmetic, one
  *             rounding to `dtype`); q_weight / q_bias / k_weight / k_bias are [head_dim] of
@@ -339,6 +340,41 @@ int come_qk_norm_rope(void *q, void *k, int dtype,
                       const void *k_weight, const void *k_bias, float eps,
                       const int64_t *positions, const void *cos_table, const void *sin_table,
                       int64_t n_pos, void *stream);
+
+/*
+ * come_attn_varlen_fwd_qp — come_attn_varlen_fwd_ws with the q half of come_qk_norm_rope applied to the query rows
+ * as the kernel loads them: q in memory is the raw projection (it is not written), k has been through
+ * come_qk_norm_rope (which skips a NULL q), and the result is bit for bit what come_attn_varlen_fwd_ws returns after
+ * come_qk_norm_rope on both - the kernel runs the same arithmetic in the same order on its query fragments.  Saves
+ * the read and the write of q in the prologue pass (half its traffic).
+ *
+ *   prologue  the q-side arguments of come_qk_norm_rope with the same meaning (weight / bias may be NULL;
+ *             positions NULL = no rotation, otherwise cos_table / sin_table [n_pos, 16] of `dtype`); pointers
+ *             16-byte aligned.  NULL makes the call identical to come_attn_varlen_fwd_ws.
+ * head_dim must be 64, and COME_ATTN_WORK_QUEUE is refused (COME_ERR_UNSUPPORTED).
+ *
+ * In the reference the prologue is a separate step of the caller (src/accelerate/common/qkv.py:31-39, called at
+ * src/accelerate/vggt/module/bias_attention.py:100-106 right in front of the operator); this entry point is for a
+ * caller that hands the q-side step to the operator.
+ */
+typedef struct come_q_prologue {
+    int apply_norm;                 /* 0 = no LayerNorm */
+    float eps;
+    const void *weight, *bias;      /* [64] of dtype, NULL = 1 resp. 0 */
+    const int64_t *positions;       /* [total, 2] (y, x), NULL = no rotation */
+    const void *cos_table, *sin_table;
+    int64_t n_pos;
+} come_q_prologue;
+int come_attn_varlen_fwd_qp(const void *q, const void *k, const void *v, int dtype,
+                            int64_t q_row_stride, int64_t q_head_stride,
+                            int64_t k_row_stride, int64_t k_head_stride,
+                            int64_t v_row_stride, int64_t v_head_stride,
+                            const int32_t *cu_seqlens, int64_t n_seq, int64_t total,
+                            int64_t n_heads, int64_t head_dim,
+                            const void *perkey_bias, int64_t max_seqlen, float softmax_scale,
+                            void *out, int64_t o_row_stride, int64_t o_head_stride,
+                            float *lse, void *work, int64_t work_bytes,
+                            const come_q_prologue *prologue, int flags, void *stream);
 
 /*
  * come_jagged_add_suffix / come_jagged_split_suffix — append `count` dense rows to every packed

@@ -80,3 +80,16 @@ def test_merged_close_to_unmerged():
     same = model(images, merger=hip_merger(0.0))
     assert same["tokens_packed"] == same["tokens_dense"]
     assert relative_l1(same["maps"], dense["maps"]) < 1e-2
+
+
+def test_deferred_q_prologue_gives_the_same_bits_end_to_end():
+    """The whole model with the q half of every attention prologue left to the attention kernel
+    (``deferred_q_prologue``): merged and unmerged forward, the same output bits as with the in-place pass."""
+    from come_amd.harness import deferred_q_prologue
+
+    model = build(256, 4, 3, 1, (1, 2))
+    images = torch.rand(1, 2, 3, 518, 518, generator=torch.Generator().manual_seed(5)).cuda()
+    for merger in (hip_merger(0.5), None):
+        two_step = model(images, merger=merger)
+        fused = model(images, merger=merger, prologue=deferred_q_prologue)
+        assert torch.equal(two_step["maps"], fused["maps"])
