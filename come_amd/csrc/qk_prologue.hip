@@ -34,6 +34,7 @@ struct QkArgs {
     const void *cos_table;        // [n_pos, 16]
     const void *sin_table;
     int64_t n_pos;
+    int groups_per_wg;            // token groups that share a workgroup (1: the groups' lanes are sliced over blockIdx.y)
 };
 
 template <int DT>
@@ -71,14 +72,23 @@ template <int DT>
 __global__ void __launch_bounds__(256) qk_norm_rope_kernel(const QkArgs a) {
     using V = Vec16<DT>;
     using C = QkChunk<DT>;
-    const int j = blockIdx.y * 256 + threadIdx.x;                 // (which, head, lane8) of this lane
     const int per_tensor = a.n_heads * 8;
     const int first = a.ptr[0] != nullptr ? 0 : 1, n_tensors = (a.ptr[0] != nullptr ? 1 : 0) + (a.ptr[1] != nullptr ? 1 : 0);
-    if (j >= n_tensors * per_tensor) return;                      // the eight lanes of a head leave together
+    const int per_group = n_tensors * per_tensor;                 // lanes that one group of tokens needs
+    // a workgroup holds a.groups_per_wg token groups side by side when one of them leaves half of it or more empty
+    // (few heads, or one tensor only), else one group per 256-thread slice
+    const int j = a.groups_per_wg > 1 ? static_cast<int>(threadIdx.x) % per_group
+                                      : static_cast<int>(blockIdx.y * 256 + threadIdx.x);       // (which, head, lane8) of this lane
+    const int64_t group = a.groups_per_wg > 1
+                              ? static_cast<int64_t>(blockIdx.x) * a.groups_per_wg + static_cast<int>(threadIdx.x) / per_group
+                              : static_cast<int64_t>(blockIdx.x);
+    const int64_t token0 = group * kRowsPerThread;
+    // (the eight lanes of a head leave together: per_group is a multiple of 8)
+    if (j >= per_group || token0 >= a.total) return;
+    if (a.groups_per_wg > 1 && static_cast<int>(threadIdx.x) / per_group >= a.groups_per_wg) return;   // lanes beyond the last whole group
     const int which = first + (j >= per_tensor ? 1 : 0);
     const int head = (j - (which - first) * per_tensor) >> 3;
     const int lane8 = j & 7;
-    const int64_t token0 = static_cast<int64_t>(blockIdx.x) * kRowsPerThread;
 
     char *row = static_cast<char *>(a.ptr[which]) +
                 (token0 * a.row_stride[which] + head * a.head_stride[which]) * V::ELEM_BYTES + lane8 * 16;
@@ -193,8 +203,10 @@ extern "C" int come_qk_norm_rope(void *q, void *k, int dtype,
     a.cos_table = cos_table;
     a.sin_table = sin_table;
     a.n_pos = n_pos;
-    const int64_t groups = ceil_div(total, kRowsPerThread);
-    const int64_t slices = ceil_div(((q != nullptr) + (k != nullptr)) * n_heads * 8, 256);
+    const int64_t per_group = ((q != nullptr) + (k != nullptr)) * n_heads * 8;
+    a.groups_per_wg = per_group <= 128 ? static_cast<int>(256 / per_group) : 1;
+    const int64_t groups = ceil_div(ceil_div(total, kRowsPerThread), a.groups_per_wg);
+    const int64_t slices = a.groups_per_wg > 1 ? 1 : ceil_div(per_group, 256);
     COME_REQUIRE(groups < (int64_t{1} << 31) && slices < 65536 && n_pos < (1 << 24), COME_ERR_UNSUPPORTED,
                  "come_qk_norm_rope: too many tokens, heads or positions for one launch");
     const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(slices));
