@@ -37,7 +37,7 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 # device copy (``--only copy``) gives for the same counters.  Each entry names the summary under profiles/ that holds
 # the run it was read from; a kernel change means a new run of the commands written there and new numbers here.
 TRAFFIC = {
-    "attn": {"bytes": int((265900 * 2.000 + 97740) * 1024), "source": "profiles/attn_fwd_c3.txt"},
+    "attn": {"bytes": int((266639 * 2.000 + 97737) * 1024), "source": "profiles/attn_fwd_c3.txt"},
     "merge": {"bytes": int((22072 * 2.000 + 25943) * 1024), "source": "profiles/merge_c2_r050.txt"},
     "unmerge": {"bytes": int((13632 * 2.000 + 43970) * 1024), "source": "profiles/unmerge_c2_r050.txt"},
 }
@@ -54,7 +54,7 @@ def parse_args():
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end aggregator leg")
     ap.add_argument("--scale-mode", choices=["auto", "exact", "folded"], default="auto",
                     help="with --only frame / stress_frames: how softmax_scale is applied (one kernel per profiler run)")
-    ap.add_argument("--only", choices=["stress_frames", "attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "prologue", "copy", "exact", "folded", "widths", "select", "e2e", "stress", "stress_e2e", "frame"], default=None,
+    ap.add_argument("--only", choices=["stress_frames", "attn", "merge", "unmerge", "pair", "dtypes", "bias", "refmerge", "prologue", "prologue_k", "copy", "exact", "folded", "widths", "select", "e2e", "stress", "stress_e2e", "frame"], default=None,
                     help="run a single kernel in a loop (for profilers); prints a short JSON line")
     return ap.parse_args()
 
@@ -505,7 +505,7 @@ def bench_bias_overhead(device):
     return out
 
 
-def bench_qk_prologue(device, rows=(25536, 43968), iters=200, warmup=20):
+def bench_qk_prologue(device, rows=(25536, 43968), iters=200, warmup=20, k_only=False):
     """q / k LayerNorm + 2-D RoPE in place on the packed ``qkv [P, 3, 16, 64]`` bf16 (one launch through the C ABI),
     over 4 rotating tensors (each launch touches 2/3 of 157 MB at P = 25 536).  Algorithmic bytes: q and k read and
     written once.  ``k_only``: the same launch with a null q (half the bytes), what remains of the pass when the q half
@@ -525,7 +525,7 @@ def bench_qk_prologue(device, rows=(25536, 43968), iters=200, warmup=20):
         pos = torch.randint(0, 38, (P, 2), device=device)
         state = {"i": 0}
 
-        def step(k_only=False):
+        def step():
             i = state["i"] = (state["i"] + 1) % 4
             q, k = sets[i][:, 0], sets[i][:, 1]
             _lib.check(lib.come_qk_norm_rope(None if k_only else q.data_ptr(), k.data_ptr(), _lib.COME_BF16, q.stride(0), q.stride(1),
@@ -534,14 +534,10 @@ def bench_qk_prologue(device, rows=(25536, 43968), iters=200, warmup=20):
                                              pos.data_ptr(), cos_t.data_ptr(), sin_t.data_ptr(), 38, stream))
 
         _, ms = time_loop(step, iters, warmup)
-        nbytes = P * 2 * H * 64 * 2 * 2
+        nbytes = P * (1 if k_only else 2) * H * 64 * 2 * 2
         gbs = nbytes / (ms / iters * 1e-3) / 1e9
-        _, ms_k = time_loop(lambda: step(True), iters, warmup)
-        gbs_k = nbytes / 2 / (ms_k / iters * 1e-3) / 1e9
         out["P=%d" % P] = {"us_per_call": round(ms / iters * 1e3, 2), "algorithmic_bytes": nbytes, "GBs": round(gbs, 1),
-                           "frac": round(gbs / PEAK_HBM_GBS, 4),
-                           "k_only": {"us_per_call": round(ms_k / iters * 1e3, 2), "algorithmic_bytes": nbytes // 2,
-                                      "GBs": round(gbs_k, 1), "frac": round(gbs_k / PEAK_HBM_GBS, 4)}}
+                           "frac": round(gbs / PEAK_HBM_GBS, 4)}
         del sets
         torch.cuda.empty_cache()
     return out
@@ -868,7 +864,9 @@ def main():
         elif args.only == "widths":
             print(json.dumps({"only": "widths", **bench_other_widths(device, args.steps, args.warmup)}))
         elif args.only == "prologue":
-            print(json.dumps({"only": "prologue", **bench_qk_prologue(device, iters=args.steps, warmup=args.warmup),
+            print(json.dumps({"only": "prologue", **bench_qk_prologue(device, iters=args.steps, warmup=args.warmup)}))
+        elif args.only == "prologue_k":
+            print(json.dumps({"only": "prologue_k", **bench_qk_prologue(device, iters=args.steps, warmup=args.warmup, k_only=True),
                               "q_half_in_attention": bench_deferred_q_prologue(device)}))
         elif args.only == "refmerge":
             print(json.dumps({"only": "refmerge", **bench_reference_merge_shapes(device)}))
@@ -936,6 +934,7 @@ def main():
         other["merge_caller_dtypes"] = bench_merge_caller_dtypes(device)
         other["reference_merge_microbench_shapes"] = bench_reference_merge_shapes(device)
         other["qk_prologue"] = bench_qk_prologue(device)
+        other["qk_prologue"]["k_only"] = bench_qk_prologue(device, k_only=True)
         other["qk_prologue"]["q_half_in_attention"] = bench_deferred_q_prologue(device)
         other["frame_attention"] = bench_frame_attention(device, w)
         other["bias_overhead"] = bench_bias_overhead(device)
