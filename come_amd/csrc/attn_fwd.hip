@@ -615,10 +615,12 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     auto finish_slot = [&](int Y, const f32x4 (&ssum)[2]) __attribute__((always_inline)) {
         // sums are not negative: if the four rows of a lane together stay within the limit, each of them does
         // (written so that a NaN counts as beyond it)
-        const f32x4 &c0 = kChain ? l_acc[0] : ssum[0];
-        const f32x4 &c1 = kChain ? l_acc[1] : ssum[1];
+        // kChain: the running sums only grow between two moves of the reference point, so one query tile is looked
+        // at per slot, each of them once per key tile (whatever the other collected in between is still in its sum)
+        const f32x4 &c0 = kChain ? l_acc[Y] : ssum[0];
+        const f32x4 &c1 = kChain ? l_acc[Y] : ssum[1];
         const float t0 = (c0[0] + c0[1]) + (c0[2] + c0[3]);
-        const float t1 = (c1[0] + c1[1]) + (c1[2] + c1[3]);
+        const float t1 = kChain ? t0 : (c1[0] + c1[1]) + (c1[2] + c1[3]);
         const bool bad = !(t0 <= kSumLimit) || !(t1 <= kSumLimit);
         if (__any(bad) || any_pending || has_delta) {
             // the asm arithmetic below reads MFMA results; the compiler cannot see that, so the wait states an
