@@ -796,9 +796,9 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
             __syncthreads();
         }
     } else {
-        for (int j = 0; j < n_tiles; ++j) {
-            const int t = ring + j;
-            const int kb = t & 3, kb1 = (t + 1) & 3, kb2 = (t + 2) & 3, kb3 = (t + 3) & 3;   // stage of tile j, j+1, ..
+        // one key tile: `kb` is the ring stage of tile j
+        auto iteration = [&](int j, int kb) __attribute__((always_inline)) {
+            const int kb1 = (kb + 1) & 3, kb2 = (kb + 2) & 3, kb3 = (kb + 3) & 3;   // stage of tile j + 1, ..
             load_bias(j + 4, kb);      // raw bias runs one more tile ahead (converted between the slots of iteration j+2)
             stage_k(j + 3, kb3);       // K(j+3) replaces K(j-1), V(j+2) replaces V(j-2): both idle since the
             stage_v(j + 2, kb2);       // last barrier; they are first read two barriers from now
@@ -818,6 +818,28 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
                 if (j == n_tiles - 1 && tl == 0) lds_claim = claim;
             }
             __syncthreads();
+        };
+        if constexpr (PERSIST || NW != 8) {
+            for (int j = 0; j < n_tiles; ++j) iteration(j, (ring + j) & 3);
+        } else {
+            // long segments (the ring starts at stage 0): four tiles per turn of the loop make every stage a constant,
+            // so that the fragment reads address LDS through their offset fields instead of through six additions
+            // per slot (+2.5 %).  The workgroups of short segments keep the plain loop: their few tiles do not repay
+            // the registers the four copies cost there.
+            int j = 0;
+            for (; j + 4 <= n_tiles; j += 4) {
+                iteration(j, 0);
+                iteration(j + 1, 1);
+                iteration(j + 2, 2);
+                iteration(j + 3, 3);
+            }
+            if (j < n_tiles) {
+                iteration(j, 0);
+                if (j + 1 < n_tiles) {
+                    iteration(j + 1, 1);
+                    if (j + 2 < n_tiles) iteration(j + 2, 2);
+                }
+            }
         }
     }
 
