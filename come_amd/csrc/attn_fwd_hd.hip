@@ -223,8 +223,7 @@ __global__ __launch_bounds__(256) void attn_fwd_hd_kernel(const AttnArgs a) {
 
     // A wavefront whose 32 queries all lie beyond the end of the segment only helps with the staging.
     const bool idle = q0 + wave_u * 32 >= L;
-    for (int j = 0; j < n_tiles; ++j) {
-        const int buf = j & 1;
+    auto iteration = [&](int j, int buf) __attribute__((always_inline)) {
         float b_next = 0.f;
         if (j + 1 < n_tiles) {
             stage(j + 1, buf ^ 1);             // that stage was last read before the previous barrier
@@ -245,7 +244,14 @@ __global__ __launch_bounds__(256) void attn_fwd_hd_kernel(const AttnArgs a) {
         if (j + 1 < n_tiles && wave_u == 0) lds_b[buf ^ 1][lane] = b_next;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+    };
+    // two tiles per turn: the LDS stage is a constant in each copy and goes into the offset fields of the reads
+    int j = 0;
+    for (; j + 2 <= n_tiles; j += 2) {
+        iteration(j, 0);
+        iteration(j + 1, 1);
     }
+    if (j < n_tiles) iteration(j, 0);
     if (idle) return;
 
     // ---- epilogue: normalise, write O (and LSE)
