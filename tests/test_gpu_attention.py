@@ -494,6 +494,29 @@ def test_full_size_c3_rows_against_oracle_rows():
         torch.testing.assert_close(lse[:, row], torch.logsumexp(scores, -1), atol=2e-3, rtol=1e-3)
 
 
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("L", [8192, 8129, 8127, 8064, 7999], ids=lambda L: f"L{L}")
+def test_long_segment_launch_with_every_remainder_of_its_four_tile_loop(L, mode):
+    """One segment that fills a round of 512-query workgroups (16 heads x 16 blocks = 256): the instantiation whose
+    key loop takes four 64-key tiles per turn.  128, 128 (one key into the last tile), 127, 126 and 125 tiles leave
+    0, 0, 3, 2 and 1 tiles behind the last full turn; rows sampled over the segment against the closed form."""
+    H = 16
+    g = torch.Generator().manual_seed(L)
+    qkv = torch.randn(L, 3, H, 64, generator=g).bfloat16()
+    bias = torch.where(torch.rand(L, generator=g) < 0.3, 2.197, 0.0).bfloat16()
+    out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), _cu([L]).to(DEV), L, perkey_bias=bias.to(DEV),
+                                                                 return_attn_probs=True, scale_mode=mode)
+    out, lse = out.float().cpu(), lse.cpu()
+    assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(lse).all())
+    q, k, v = qkv.float().unbind(1)
+    for row in [0, 33, 511, 512, 4000, L - 513, L - 65, L - 64, L - 1]:
+        scores = torch.einsum("hd,khd->hk", q[row], k) * 0.125 + bias.float()[None]
+        ref = torch.einsum("hk,khd->hd", torch.softmax(scores, -1), v)
+        diff = (out[row] - ref).abs()
+        assert float(diff.max()) <= MAX_ABS and float(diff.mean()) <= MEAN_ABS, (row, float(diff.max()))
+        torch.testing.assert_close(lse[:, row], torch.logsumexp(scores, -1), atol=4e-3, rtol=1e-3)
+
+
 BORDER_LENGTHS = [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 300, 511, 512, 513, 767, 769, 1023, 1025]
 
 
