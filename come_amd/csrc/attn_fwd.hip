@@ -848,6 +848,17 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     // fp16) within one 32-key step leaves an infinite or saturated probability behind.  The wavefront that saw such a
     // row sum said so in front of the loop's last barrier, and the workgroup then computes its block once more with the textbook running maximum
     // (one tile at a time, no pipelining: slow, exact for any scores, and never taken by ordinary attention logits).
+    if constexpr (kChain) {
+        // The checks inside the loop look at one query tile per slot: what the last slot added to the other one is
+        // looked at here (only a sum beyond the hard limit matters now), and the wavefront's word is said once more.
+        if (!idle) {
+            const float ta = (l_acc[0][0] + l_acc[0][1]) + (l_acc[0][2] + l_acc[0][3]);
+            const float tb = (l_acc[1][0] + l_acc[1][1]) + (l_acc[1][2] + l_acc[1][3]);
+            overflowed = overflowed || __any(!(ta <= Range<DT>::kHardLimit) || !(tb <= Range<DT>::kHardLimit));
+            if (lane == 0) lds_ref[wave] = overflowed ? 1.f : 0.f;
+        }
+        __syncthreads();
+    }
     bool again = false;
 #pragma unroll
     for (int w = 0; w < NW; ++w) again = again || lds_ref[w] != 0.f;

@@ -270,6 +270,32 @@ def test_late_key_just_inside_the_float_range_with_large_values(jump, mode):
     torch.testing.assert_close(lse.cpu(), ref_lse, atol=2e-2 if mode == "folded" else 5e-3, rtol=1e-3)
 
 
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("where", [1, 2, 31, 33, 40, 64, 65], ids=lambda w: f"last-{w}")
+def test_key_beyond_the_range_in_the_last_tile_of_a_segment(where, mode):
+    """The key that leaves the range of the stored probabilities is one of the last 65 keys of its segment (last
+    key, last half-tile, the half-tile before it, the tile before), in a segment that ends on a tile border, one that
+    ends one key behind it and a short second one: the sums of the last slots are looked at behind the loop."""
+    lens, H = [1536, 1473, 100], 2
+    P = sum(lens)
+    g = torch.Generator().manual_seed(where)
+    qkv = torch.randn(P, 3, H, 64, generator=g).bfloat16()
+    bias = torch.zeros(P)
+    end = 0
+    for L in lens:
+        end += L
+        bias[end - where] = 150.0
+    bias = bias.bfloat16()
+    cu = _cu(lens)
+    ref, ref_lse = oracle.biased_varlen_attention(qkv, cu, bias)
+    out, lse, _ = flash_attn_varlen_qkvpacked_func_w_perkey_bias(qkv.to(DEV), cu.to(DEV), max(lens),
+                                                                 perkey_bias=bias.to(DEV), return_attn_probs=True,
+                                                                 scale_mode=mode)
+    assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(lse).all())
+    torch.testing.assert_close(out.float().cpu(), ref, atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(lse.cpu(), ref_lse, atol=2e-2 if mode == "folded" else 5e-3, rtol=1e-3)
+
+
 def test_key_beyond_the_range_inside_a_key_split_piece():
     """The same situation in a launch whose last query blocks are cut along the keys (long single segment with a work
     buffer): the piece that meets the key computes its share again; pieces are combined as usual."""
