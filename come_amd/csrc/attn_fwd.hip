@@ -1252,7 +1252,7 @@ static void *static_work_pointer() {
     return known[dev];
 }
 
-// Shared body of the three entry points.  static_work: the buffer is the library's own fixed-size array; a launch
+// Shared body of the attention entry points.  static_work: the buffer is the library's own fixed-size array; a launch
 // that needs more is an error instead of a launch without the key split.
 static int attn_varlen_fwd_impl(const void *q, const void *k, const void *v, int dtype, int64_t q_row_stride,
                                 int64_t q_head_stride, int64_t k_row_stride, int64_t k_head_stride,

@@ -48,6 +48,29 @@ def test_version_and_error_string():
     assert lib.come_select_work_bytes(1, 16, 37, 37, 3, 3) >= 16 * 144 * 4
 
 
+def test_q_prologue_entry_point_checks_its_descriptor_on_the_host():
+    """come_attn_varlen_fwd_qp refuses what it cannot do before anything is launched (the pointers are never followed)."""
+    lib = _lib.load()
+    fake = 0x10000                                   # an aligned address that is not dereferenced
+
+    def call(head_dim, desc, flags):
+        row = 3 * 16 * head_dim
+        return lib.come_attn_varlen_fwd_qp(fake, fake, fake, _lib.COME_BF16, row, head_dim, row, head_dim, row, head_dim,
+                                           fake, 1, 10, 16, head_dim, None, 10, 0.125, fake, 16 * head_dim, head_dim, None,
+                                           None, 0, desc, flags, None)
+
+    norm = _lib.QPrologue(1, 1e-5, None, None, None, None, None, 0)
+    assert call(128, ctypes.byref(norm), 0) == 2 and b"head_dim must be 64" in lib.come_last_error()
+    assert call(64, ctypes.byref(norm), _lib.COME_ATTN_WORK_QUEUE) == 2 and b"COME_ATTN_WORK_QUEUE" in lib.come_last_error()
+    assert call(64, ctypes.byref(_lib.QPrologue(1, -1.0, None, None, None, None, None, 0)), 0) == 1
+    assert b"eps" in lib.come_last_error()
+    assert call(64, ctypes.byref(_lib.QPrologue(0, 0.0, None, None, fake, None, None, 0)), 0) == 1
+    assert b"tables" in lib.come_last_error()
+    assert call(64, ctypes.byref(_lib.QPrologue(1, 1e-5, fake + 2, None, None, None, None, 0)), 0) == 1
+    assert b"aligned" in lib.come_last_error()
+    assert call(64, ctypes.byref(norm), 4) == 1 and b"flags" in lib.come_last_error()
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "_lib", None)
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libcome_hip.so")
