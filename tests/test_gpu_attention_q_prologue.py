@@ -116,6 +116,19 @@ def test_key_split_tail_of_a_long_launch():
     assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)
 
 
+def test_same_bits_at_the_size_of_the_benchmark_workload():
+    """16 heads, two packed sequences of 25 536 and 21 848 rows (the 512-query workgroups with their four-tile loop,
+    full rounds and a key-split tail)."""
+    dtype = torch.bfloat16
+    lens, H = [25536, 21848], 16
+    qkv, (qn, kn), pos, bias = _inputs(lens, H, dtype, seed=1)
+    (out_a, lse_a, t_a), (out_b, lse_b, t_b) = _both_ways(qkv, qn.cuda(), kn.cuda(), RotaryPositionEmbedding2D(100.0), pos, bias,
+                                                         lens, dtype)
+    assert torch.equal(t_a[:, 1], t_b[:, 1])
+    assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)
+    assert bool(torch.isfinite(out_b).all())
+
+
 @torch.no_grad()
 def test_against_the_oracle():
     """Prologue and attention of the oracle on the raw tensor against the deferred path, at the operator's tolerance.
