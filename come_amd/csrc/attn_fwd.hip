@@ -602,7 +602,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
             }
     };
 
-    // End of a slot.  Steady state: add the half-tile row sums.  The scores the slot built (buffer Y) are
+    // End of a slot.  Steady state: the range check (fp16: and adding the slot's row sums).  The scores the slot built (buffer Y) are
     // relative to m_base; rows whose reference point differs from it are corrected here (rare: it takes a
     // wavefront whose rows differ by more than 2^kMaxGap in magnitude, or a row sum that left the safe range).
     // When a row sum leaves the safe range the reference point of the row moves up by a power of two, 2^shift:
@@ -611,7 +611,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     //    which are relative to the old reference, have been accumulated.
     float o_pending[2] = {1.f, 1.f};
     bool any_pending = false;                  // wave-uniform
-    bool overflowed = false;                   // wave-uniform: some half-tile row sum exceeded kHardLimit
+    bool overflowed = false;                   // wave-uniform: some row sum exceeded kHardLimit
     auto finish_slot = [&](int Y, const f32x4 (&ssum)[2]) __attribute__((always_inline)) {
         // sums are not negative: if the four rows of a lane together stay within the limit, each of them does
         // (written so that a NaN counts as beyond it)
