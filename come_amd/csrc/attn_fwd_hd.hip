@@ -10,8 +10,9 @@
 // one barrier per tile.  Scores are computed transposed (S^T = K Q^T) so that the probabilities
 // leave the accumulators as the B operand of O^T += V^T P^T, as in the 64-wide kernel.
 //
-// Softmax: the scale and the bias are applied to every fp32 score by one fused multiply-add, as the
-// reference does (softmax.h:76-88, flash_fwd_kernel.h:30-55), in log2 units.  The reference point of
+// Softmax: the score accumulators start from bias / scale, so that the MFMAs deliver q . k + bias / scale as the
+// reference forms it (flash_fwd_kernel.h:30-55), and one fused multiply-add per score applies the scale and
+// subtracts the row's reference point in front of the exponential (softmax.h:76-88), in log2 units.  The reference point of
 // a row is a running maximum that is only moved when a half-tile's maximum exceeds it by more than
 // 2^8: probabilities stay below 2^8 (exact in both 16-bit types), the result is the same up to
 // rounding, and the output accumulators are rescaled a few times per row instead of every 32 keys.
@@ -47,7 +48,7 @@ __global__ __launch_bounds__(256) void attn_fwd_hd_kernel(const AttnArgs a) {
     constexpr float kLog2e = 1.4426950408889634f;
     __shared__ __attribute__((aligned(1024))) uint16_t lds_k[2][kBlockN * D];
     __shared__ __attribute__((aligned(1024))) uint16_t lds_v[2][kBlockN * D];
-    __shared__ __attribute__((aligned(16))) float lds_b[2][kBlockN];     // bias log2(e), -inf beyond the segment
+    __shared__ __attribute__((aligned(16))) float lds_b[2][kBlockN];     // bias / softmax_scale, -inf beyond the segment
 
     // workgroup i runs on XCD i % 8: the query blocks of one (segment, head) unit stay on one XCD
     const int xcd = blockIdx.x & 7;
@@ -116,11 +117,13 @@ __global__ __launch_bounds__(256) void attn_fwd_hd_kernel(const AttnArgs a) {
             dma_b128(v_seg, vo, lds_address(&lds_v[buf][(kDma * wave_u + i) * 512]));
         }
     };
-    // bias of a tile's 64 keys in log2 units (wavefront 0, lane = key)
+    // What the scores of a tile's 64 keys start from (wavefront 0, lane = key): bias / softmax_scale, as the
+    // reference adds it to the raw scores (flash_fwd_kernel.h:46-50); -inf beyond the end of the segment
+    const float inv_c = 1.0f / a.scale_log2;
     auto bias_of = [&](int tile) __attribute__((always_inline)) -> float {
         const int key = tile * kBlockN + lane;
         if (key >= L) return -INFINITY;
-        return a.bias ? E::to_f32(a.bias[seq_start + key]) * kLog2e : 0.f;
+        return a.bias ? E::to_f32(a.bias[seq_start + key]) * kLog2e * inv_c : 0.f;
     };
 
     // ---- LDS read offsets (in elements) of this lane
@@ -152,10 +155,19 @@ __global__ __launch_bounds__(256) void attn_fwd_hd_kernel(const AttnArgs a) {
                                : u32x4{0u, 0u, 0u, 0u};
     const int owner_base = (16 * (lane & 15) + 4 * (lane >> 4)) & 31;     // element j of l_acc belongs to query owner_base + j
 
-    // k-step ks of the scores of half-tile `half` of the K tile in `buf`
+    // k-step ks of the scores of half-tile `half` of the K tile in `buf`; the accumulator starts from the bias terms
+    // of the lane's 16 keys (rows 8 g + 4 h + e of the half-tile), so that q . k + bias / scale leaves the MFMAs
     auto score_step = [&](f32x16 &s, int buf, int half, int ks) __attribute__((always_inline)) {
         const u32x4 kf = *reinterpret_cast<const u32x4 *>(&lds_k[buf][k_rd[ks] + 32 * half * D]);
-        s = E::mfma(kf, qf[ks], ks == 0 ? zero16 : s);
+        if (ks == 0) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 bq = *reinterpret_cast<const f32x4 *>(&lds_b[buf][32 * half + 8 * g + 4 * h]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) s[4 * g + e] = bq[e];
+            }
+        }
+        s = E::mfma(kf, qf[ks], s);
     };
     // MFMA m of O^T += V^T P^T for half-tile `half` of the V tile in `buf` (m = 16-key step x output tile)
     auto pv_step = [&](const u32x4 (&p)[2], int buf, int half, int m) __attribute__((always_inline)) {
@@ -169,18 +181,10 @@ __global__ __launch_bounds__(256) void attn_fwd_hd_kernel(const AttnArgs a) {
     // Scores of one half-tile -> probabilities (B operands p[16-key step]).  `mfma(m)` issues the m-th of kKSteps
     // (= 2 kDTiles) independent MFMAs of the neighbouring half-tile, spread between the exponentials.
     auto softmax_step = [&](const f32x16 &s, int buf, int half, u32x4 (&p)[2], auto &&mfma) __attribute__((always_inline)) {
-        float x[16];
         float mx = -INFINITY;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const f32x4 bq = *reinterpret_cast<const f32x4 *>(&lds_b[buf][32 * half + 8 * g + 4 * h]);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                x[4 * g + e] = __builtin_fmaf(s[4 * g + e], a.scale_log2, bq[e]);
-                mx = fmaxf(mx, x[4 * g + e]);
-            }
-        }
-        mx = max_across_halves(mx);
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[e]);
+        mx = max_across_halves(mx) * a.scale_log2;               // the scale is positive: the maximum commutes with it
         // A reference point that moves rescales the row sum now and the output at the end of the step, behind the
         // P V MFMAs issued in between: their probabilities are relative to the old reference point.
         const bool move = mx > m_ref + kRefSlack;              // (also the first keys of a row: m_ref = -inf)
@@ -192,7 +196,7 @@ __global__ __launch_bounds__(256) void attn_fwd_hd_kernel(const AttnArgs a) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) l_acc[j] *= __shfl(down, owner_base + j);
         }
-        const float ref = m_ref == -INFINITY ? 0.f : m_ref;     // a row that has seen masked keys only
+        const float neg_ref = m_ref == -INFINITY ? 0.f : -m_ref;   // (a row that has seen masked keys only: 0)
 #pragma unroll
         for (int w = 0; w < 8; ++w) {
             if (kKSteps >= 8) {
@@ -201,8 +205,8 @@ __global__ __launch_bounds__(256) void attn_fwd_hd_kernel(const AttnArgs a) {
             } else if (w % (8 / kKSteps) == 0) {
                 mfma(w / (8 / kKSteps));
             }
-            const uint32_t pw = E::pack2_prob(__builtin_amdgcn_exp2f(x[2 * w] - ref),
-                                              __builtin_amdgcn_exp2f(x[2 * w + 1] - ref));
+            const uint32_t pw = E::pack2_prob(__builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * w], a.scale_log2, neg_ref)),
+                                              __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * w + 1], a.scale_log2, neg_ref)));
             p[w >> 2][w & 3] = pw;
             if (w == 3) l_acc = E::mfma16(p[0], ones_sel, l_acc);
         }
